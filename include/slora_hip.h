@@ -1,0 +1,145 @@
+/*
+ * slora_hip.h -- C ABI of libslora_hip.so: heterogeneous multi-LoRA batching
+ * over a unified paged adapter pool, for AMD MI355X (gfx950).
+ *
+ * Every pointer is a DEVICE pointer unless stated otherwise.  Nothing is
+ * retained after a call returns; no call allocates, frees or synchronises.
+ * Kernels are enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ * default stream).  Every function returns SLORA_OK or a negative SLORA_ERR_*
+ * code; slora_strerror() gives the message.  Shape checks happen on the host
+ * before anything is launched; indices read on the device (adapter ids, page
+ * ids) are range-checked against n_adapters / n_loc / n_pages and a token or
+ * row whose index is out of range is skipped instead of faulting.
+ *
+ * Pool layout (reference: slora/common/mem_allocator.py:229-234,
+ * slora/models/peft/layer_weights/lora_layer_weight.py:84-93): `w` is one
+ * layer's buffer of `n_pages` pages of `page_elems` 16-bit elements.  An
+ * adapter a of rank r owns the 4r page ids a_loc[a_start[a] .. +4r), a_len[a]
+ * = 4r, grouped by projection p in (q,k,v,o):
+ *   A side (key_buffer):   page a_loc[a_start[a] + p*r + j] = column j of A_p
+ *                          (h_in elements).
+ *   B side (value_buffer): the (h_out, r) row-major matrix B_p^T laid end to
+ *                          end over pages a_loc[a_start[a] + p*r + 0..): element
+ *                          (n, d) is at flat index n*r + d, page flat /
+ *                          page_elems, offset flat % page_elems.
+ * The reference ties page_elems to h_in (shrink) / h_out (expand); here it is
+ * explicit so an output narrower than a page (grouped-query k/v) works.
+ */
+#ifndef SLORA_HIP_H
+#define SLORA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLORA_VERSION 100 /* 0.1.0 */
+
+#define SLORA_API __attribute__((visibility("default")))
+
+/* storage types of x / y / w / scales */
+#define SLORA_DTYPE_F16 0
+#define SLORA_DTYPE_BF16 1
+#define SLORA_DTYPE_F32 2 /* scales only */
+
+#define SLORA_OK 0
+#define SLORA_ERR_NULL_POINTER -1  /* a required pointer is NULL */
+#define SLORA_ERR_BAD_DTYPE -2     /* dtype is not F16/BF16 (scales: F16/BF16/F32) */
+#define SLORA_ERR_BAD_SHAPE -3     /* negative size, qkvo outside 0..3, stride too small */
+#define SLORA_ERR_UNSUPPORTED -4   /* "No suitable kernel": width not a multiple of 8, rank above 512, ... */
+#define SLORA_ERR_ALIGNMENT -5     /* a buffer the kernels read 16 bytes at a time is not 16-byte aligned */
+#define SLORA_ERR_LAUNCH -6        /* the HIP runtime refused the launch */
+
+#define SLORA_MAX_RANK 512
+
+SLORA_API int slora_version(void);
+SLORA_API const char* slora_strerror(int code);
+
+/* Index tables shared by every entry point
+ * (reference: slora/server/router/model_infer/infer_adapter.py:11-24). */
+typedef struct slora_tables {
+  const int64_t* a_start; /* [n_adapters] offset of the adapter's block in a_loc */
+  const int64_t* a_len;   /* [n_adapters] 4 * rank */
+  const int64_t* a_loc;   /* [n_loc]      page ids */
+  int64_t n_adapters;
+  int64_t n_loc;
+} slora_tables;
+
+/* Decode shrink.  Replaces dispatch_bgmv with h_in >= h_out
+ * (slora/csrc/lora_ops.cc:76-126 -> bgmv_multi_lora_rank_shrink_kernel,
+ * slora/csrc/bgmv/bgmv_impl.cuh:14-149).
+ *   y[b, j] = T( sum_k f32(w[page(a,p,j), k]) * f32(x[b, k]) ),  j < min(r_a, y_cols)
+ * with a = bins[b], r_a = a_len[a]/4, p = qkvo.  Columns j >= r_a are left
+ * untouched, nothing is scaled.  x is [batch, h_in] contiguous, y is
+ * [batch, y_cols] contiguous. */
+SLORA_API int slora_bgmv_shrink(void* y, const void* x, const void* w, const slora_tables* tables,
+                      const int64_t* bins, int64_t batch, int64_t h_in, int64_t y_cols,
+                      int64_t page_elems, int64_t n_pages, int qkvo, int dtype, void* stream);
+
+/* Decode expand.  Replaces dispatch_bgmv with h_in < h_out
+ * (slora/csrc/lora_ops.cc:76-126 -> bgmv_multi_lora_rank_expand_kernel,
+ * slora/csrc/bgmv/bgmv_impl.cuh:152-208).
+ *   y[b, n] = T( y[b, n] + T( sum_{d < min(r_a, x_cols)} f32(Bt[n*r_a + d]) * f32(x[b, d]) * f32(scales[a]) ) )
+ * x is [batch, x_cols] contiguous, y is [batch, h_out] contiguous.  `scales`
+ * is read in ITS OWN type scales_dtype (the reference reinterprets the fp16
+ * scaling table as bf16 on the bf16 path, lora_ops.cc:118). */
+SLORA_API int slora_bgmv_expand(void* y, const void* x, const void* w, const slora_tables* tables,
+                      const int64_t* bins, const void* scales, int scales_dtype, int64_t batch,
+                      int64_t x_cols, int64_t h_out, int64_t page_elems, int64_t n_pages,
+                      int qkvo, int dtype, void* stream);
+
+/* Decode shrink of q, k and v in ONE launch: the three calls of
+ * slora/models/peft/lora_unordered_batch_infer.py:267-270, 287-290, 307-310
+ * read the same x, so x is staged once.  y_q/y_k/y_v are three [batch, y_cols]
+ * buffers; semantics per projection are those of slora_bgmv_shrink with
+ * qkvo = 0, 1, 2. */
+SLORA_API int slora_bgmv_shrink_qkv(void* y_q, void* y_k, void* y_v, const void* x, const void* w,
+                          const slora_tables* tables, const int64_t* bins, int64_t batch,
+                          int64_t h_in, int64_t y_cols, int64_t page_elems, int64_t n_pages,
+                          int dtype, void* stream);
+
+/* Decode expand of q, k and v in ONE launch (the calls of
+ * lora_unordered_batch_infer.py:271-273, 291-295, 311-315).  x_* are the three
+ * [batch, x_cols] shrink outputs, y_* are [batch, h_out_*] with their own
+ * widths (k/v may be narrower than q). */
+SLORA_API int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void* x_q, const void* x_k,
+                          const void* x_v, const void* w, const slora_tables* tables,
+                          const int64_t* bins, const void* scales, int scales_dtype,
+                          int64_t batch, int64_t x_cols, int64_t h_out_q, int64_t h_out_k,
+                          int64_t h_out_v, int64_t page_elems, int64_t n_pages, int dtype,
+                          void* stream);
+
+/* Prefill (segmented) shrink.  Replaces lora_get_qkvo_fwd_shrink + _shrink_fwd_kernel
+ * (slora/models/peft/triton_kernel/lora/lora_prefill.py:139-164, 57-102).
+ * Request i owns token rows b_start_loc[i] + [0, b_seq_len[i]) and uses
+ * adapter a = b_indicies[i]:
+ *   o[row, j] = T( sum_k f32(x[row, k]) * f32(w[page(a,p,j), k]) )  for j < r_a
+ *   o[row, j] = 0                                                    for r_a <= j < max_rank
+ * x, w, o are addressed with element strides (row stride, and unit column
+ * stride required). */
+SLORA_API int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables* tables,
+                      const int32_t* b_start_loc, const int32_t* b_seq_len,
+                      const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
+                      int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride,
+                      int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
+                      int dtype, void* stream);
+
+/* Prefill (segmented) expand.  Replaces lora_get_qkvo_fwd_expand + _expand_fwd_kernel
+ * (lora_prefill.py:105-136, 10-54).
+ *   o[row, n] = T( f32(o[row, n]) + (sum_{d < r_a} f32(x[row, d]) * f32(Bt[n*r_a + d])) * f32(scales[a]) )
+ * `feat_out` is both the output width and the page width, as in the reference
+ * (BLOCK_DMODEL, lora_prefill.py:42-43) unless page_elems > 0 overrides the
+ * page width. */
+SLORA_API int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables* tables,
+                      const void* scales, int scales_dtype, const int32_t* b_start_loc,
+                      const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests,
+                      int64_t max_input_len, int64_t n_tokens, int64_t feat_out,
+                      int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
+                      int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
+                      int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLORA_HIP_H */

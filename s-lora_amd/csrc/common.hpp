@@ -1,0 +1,181 @@
+// Device helpers shared by the decode (BGMV) and prefill (segmented GEMM)
+// kernels.  gfx950 only: 64-lane wavefronts, DPP row operations, 16-byte
+// global loads.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "slora_hip.h"
+
+namespace slora {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+// ---- storage types ---------------------------------------------------------
+// A storage type turns one 32-bit word holding two 16-bit elements into two
+// floats, and rounds a float back to 16 bits (round-to-nearest-even).
+struct F16 {
+  static __device__ __forceinline__ float lo(uint32_t v) { return (float)__builtin_bit_cast(f16x2, v).x; }
+  static __device__ __forceinline__ float hi(uint32_t v) { return (float)__builtin_bit_cast(f16x2, v).y; }
+  static __device__ __forceinline__ float to_float(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+  }
+  // y + d with both operands of the storage type, one rounding
+  static __device__ __forceinline__ uint16_t add(uint16_t y, uint16_t d) {
+    _Float16 s = __builtin_bit_cast(_Float16, y) + __builtin_bit_cast(_Float16, d);
+    return __builtin_bit_cast(uint16_t, s);
+  }
+};
+
+struct BF16 {
+  static __device__ __forceinline__ float lo(uint32_t v) { return __uint_as_float(v << 16); }
+  static __device__ __forceinline__ float hi(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
+  static __device__ __forceinline__ float to_float(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+  static __device__ __forceinline__ uint16_t add(uint16_t y, uint16_t d) {
+    // the sum of two bf16 values is exact in float unless their exponents are
+    // more than 16 apart, where the smaller one cannot move the rounding
+    return from_float(to_float(y) + to_float(d));
+  }
+};
+
+// scale table element -> float, in the table's own type
+__device__ __forceinline__ float load_scale(const void* scales, int scales_dtype, int64_t a) {
+  if (scales_dtype == SLORA_DTYPE_F32) return ((const float*)scales)[a];
+  uint16_t v = ((const uint16_t*)scales)[a];
+  return scales_dtype == SLORA_DTYPE_F16 ? F16::to_float(v) : BF16::to_float(v);
+}
+
+// ---- 16-byte accesses ------------------------------------------------------
+__device__ __forceinline__ u32x4 ldg16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ u32x4 zero16() { return u32x4{0u, 0u, 0u, 0u}; }
+
+// acc += sum_i f32(w_i) * f32(x_i) over the 8 elements of two 16-byte vectors
+template <typename T>
+__device__ __forceinline__ float dot8(u32x4 w, u32x4 x, float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    acc = __builtin_fmaf(T::lo(w[i]), T::lo(x[i]), acc);
+    acc = __builtin_fmaf(T::hi(w[i]), T::hi(x[i]), acc);
+  }
+  return acc;
+}
+
+// acc += sum_i f32(w_i) * xs[i] with xs already in float
+template <typename T>
+__device__ __forceinline__ float dot8f(u32x4 w, const float (&xs)[8], float acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    acc = __builtin_fmaf(T::lo(w[i]), xs[2 * i], acc);
+    acc = __builtin_fmaf(T::hi(w[i]), xs[2 * i + 1], acc);
+  }
+  return acc;
+}
+
+// ---- cross-lane sums -------------------------------------------------------
+// DPP controls: quad_perm(a,b,c,d) = a | b<<2 | c<<4 | d<<6; 0x141 = row_half_mirror,
+// 0x140 = row_mirror.  After xor-1 and xor-2 every quad is uniform, so the two
+// mirrors act as xor-4 and xor-8.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+  return v + __int_as_float(o);
+}
+
+// Sum over aligned groups of G lanes (G a power of two <= 64); every lane of
+// a group ends up holding the group's sum.
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  if (G >= 2) v = dpp_add<0xB1>(v);   // quad_perm(1,0,3,2)
+  if (G >= 4) v = dpp_add<0x4E>(v);   // quad_perm(2,3,0,1)
+  if (G >= 8) v = dpp_add<0x141>(v);  // row_half_mirror
+  if (G >= 16) v = dpp_add<0x140>(v); // row_mirror
+  if (G >= 32) v += __shfl_xor(v, 16, 64);
+  if (G >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// Sum over the whole wavefront, result valid in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group_sum<16>(v);
+  int iv = __float_as_int(v);
+  float a = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+  float b = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+  float c = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+  float d = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+  return (a + b) + (c + d);
+}
+
+// ---- tokens that share an adapter -----------------------------------------
+// A workgroup is launched for every token b.  Tokens with the same adapter
+// are processed together so the adapter's pages are read once: the tokens
+// whose bins equal `a` are numbered in order, cut into runs of `tt`, and the
+// first token of each run ("leader") does the run's work.  Returns the number
+// of tokens in b's run if b leads it (their indices in s_members[0..n)), else
+// 0.  Must be called by all NT threads of the block; s_masks holds NT/64
+// words.  The caller synchronises before reading s_members.
+template <int NT>
+__device__ __forceinline__ int find_run(const int64_t* __restrict__ bins, int64_t batch, int b, int64_t a,
+                                        int tt, uint64_t* s_masks, int* s_members) {
+  constexpr int NW = NT / kWave;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int total = 0;   // matches in chunks already processed
+  int pos_b = -1;  // b's number among the matches, once known
+  for (int64_t base = 0; base < batch; base += NT) {
+    const int64_t t = base + tid;
+    const bool m = t < batch && bins[t] == a;
+    const uint64_t ballot = __ballot(m);
+    if (base != 0) __syncthreads();  // previous chunk's masks fully consumed
+    if (lane == 0) s_masks[wave] = ballot;
+    __syncthreads();
+    int pre = total, chunk_total = 0, pre_b = total;
+    const int bw = (int)((b - base) >> 6), bl = (int)((b - base) & 63);
+    const bool b_here = b >= base && b < base + NT;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+      const uint64_t mk = s_masks[w];
+      const int pc = __popcll(mk);
+      if (w < wave) pre += pc;
+      if (b_here) {
+        if (w < bw) pre_b += pc;
+        if (w == bw) pre_b += __popcll(mk & ((1ull << bl) - 1ull));
+      }
+      chunk_total += pc;
+    }
+    pre += __popcll(ballot & ((1ull << lane) - 1ull));
+    if (b_here) {
+      pos_b = pre_b;
+      if (pos_b % tt != 0) return 0;  // uniform: every thread computed the same pos_b
+    }
+    if (pos_b >= 0 && m) {
+      const int k = pre - pos_b;
+      if (k >= 0 && k < tt) s_members[k] = (int)t;
+    }
+    total += chunk_total;
+    if (pos_b >= 0 && total - pos_b >= tt) break;
+  }
+  const int n = total - pos_b;
+  return n < tt ? n : tt;
+}
+
+// blockIdx -> (token, block-within-token).  Consecutive workgroup ids go to
+// the 8 XCDs in turn, each with its own L2; this mapping keeps all blocks of
+// one token on one XCD so its activations and tables are fetched by one L2.
+__device__ __forceinline__ void map_block(uint32_t id, uint32_t blocks_per_token, int& token, int& blk) {
+  const uint32_t xcd = id & 7u, slot = id >> 3;
+  const uint32_t grp = slot / blocks_per_token;
+  blk = (int)(slot - grp * blocks_per_token);
+  token = (int)(grp * 8u + xcd);
+}
+
+}  // namespace slora

@@ -1,0 +1,500 @@
+// Prefill-time segmented gather-GEMM over the paged adapter pool.
+//
+// A request owns a run of consecutive token rows and one adapter.  Shrink is
+// [tokens x H] . [H x r] with the r weight rows gathered page by page; expand
+// is [tokens x r] . [r x H_out] accumulated into the output, with B^T laid end
+// to end over the adapter's pages.  Both contractions run on the matrix cores
+// (v_mfma_f32_16x16x32 f16/bf16, float accumulate); both operands are
+// K-contiguous in memory, so MFMA fragments are plain 16-byte global loads.
+//
+// Replaces slora/models/peft/triton_kernel/lora/lora_prefill.py:10-164 of the
+// reference.
+
+#include "common.hpp"
+#include "cabi_util.hpp"
+
+namespace slora {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <typename T>
+__device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c);
+template <>
+__device__ __forceinline__ f32x4 mfma16<F16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ f32x4 mfma16<BF16>(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0,
+                                                 0);
+}
+
+struct SegTables {
+  const int64_t* a_start;
+  const int64_t* a_len;
+  const int64_t* a_loc;
+  const int32_t* b_start_loc;
+  const int32_t* b_seq_len;
+  const int64_t* b_indicies;
+  int64_t n_adapters, n_loc, n_pages;
+  int n_requests, n_tokens;
+};
+
+__device__ __forceinline__ int64_t seg_page(const SegTables& t, int64_t li) {
+  if ((uint64_t)li >= (uint64_t)t.n_loc) return -1;
+  const int64_t page = t.a_loc[li];
+  return (uint64_t)page < (uint64_t)t.n_pages ? page : -1;
+}
+
+// Request `req`: its adapter, rank, first row and row count clipped to the
+// buffers.  False if the request has nothing to do.
+__device__ __forceinline__ bool seg_lookup(const SegTables& t, int req, int64_t& a, int& r, int& row0, int& rows) {
+  a = t.b_indicies[req];
+  if ((uint64_t)a >= (uint64_t)t.n_adapters) return false;
+  r = (int)(t.a_len[a] >> 2);
+  row0 = t.b_start_loc[req];
+  rows = t.b_seq_len[req];
+  if (row0 < 0 || rows <= 0) return false;
+  if (row0 >= t.n_tokens) return false;
+  if (rows > t.n_tokens - row0) rows = t.n_tokens - row0;
+  return true;
+}
+
+// ---------------------------------------------------------------------------
+// shrink
+// ---------------------------------------------------------------------------
+struct SegShrinkArgs {
+  void* o;
+  const void* x;
+  const void* w;
+  SegTables t;
+  int64_t x_stride, w_stride, o_stride;  // elements per row
+  int h_in, max_rank, qkvo, m_tiles;
+  int vec_ok;  // every row start is 16-byte aligned and h_in % 8 == 0
+};
+
+constexpr int kShrThreads = 512;
+constexpr int kShrWaves = kShrThreads / kWave;  // K is split over the 8 wavefronts
+constexpr int kShrTM = 32;                      // token rows per workgroup
+constexpr int kShrNB = 64;                      // rank columns per pass
+constexpr int kShrLd = kShrNB + 4;              // LDS row pitch (floats) -> conflict-free C-tile stores
+
+// Element-wise fallback for layouts the vector path cannot read.
+template <typename T>
+__device__ void shrink_generic(const SegShrinkArgs& p, int r_eff, int64_t base_li, int row0, int m0, int m_cnt) {
+  const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* w = reinterpret_cast<const uint16_t*>(p.w);
+  uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
+  for (int idx = threadIdx.x; idx < m_cnt * p.max_rank; idx += kShrThreads) {
+    const int m = idx / p.max_rank, j = idx - m * p.max_rank;
+    const int64_t row = row0 + m0 + m;
+    float acc = 0.f;
+    if (j < r_eff) {
+      const int64_t page = seg_page(p.t, base_li + j);
+      if (page >= 0) {
+        const uint16_t* wr = w + page * p.w_stride;
+        const uint16_t* xr = x + row * p.x_stride;
+        for (int k = 0; k < p.h_in; ++k) acc = __builtin_fmaf(T::to_float(xr[k]), T::to_float(wr[k]), acc);
+      }
+    }
+    o[row * p.o_stride + j] = T::from_float(acc);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrinkArgs p) {
+  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int req = blockIdx.x / p.m_tiles;
+  const int m0 = (blockIdx.x - req * p.m_tiles) * kShrTM;
+  int64_t a;
+  int r, row0, rows;
+  if (!seg_lookup(p.t, req, a, r, row0, rows)) return;
+  if (m0 >= rows) return;
+  const int m_cnt = rows - m0 < kShrTM ? rows - m0 : kShrTM;
+  const int r_eff = r < p.max_rank ? r : p.max_rank;
+  const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
+  if (!p.vec_ok) {
+    shrink_generic<T>(p, r_eff, base_li, row0, m0, m_cnt);
+    return;
+  }
+
+  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
+  uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
+  const int lr = lane & 15, lg = lane >> 4;  // fragment row / k-group of this lane
+  const int ksteps = (p.h_in + 31) >> 5;     // 32 k per MFMA
+
+  // token rows of the two A fragments (clamped; rows past the end contribute
+  // nothing because their results are never stored)
+  const uint16_t* xrow[2];
+#pragma unroll
+  for (int f = 0; f < 2; ++f) {
+    int m = f * 16 + lr;
+    if (m >= m_cnt) m = m_cnt - 1;
+    xrow[f] = xg + (int64_t)(row0 + m0 + m) * p.x_stride;
+  }
+
+  for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
+    const int nb_cnt = p.max_rank - nb0 < kShrNB ? p.max_rank - nb0 : kShrNB;
+    if (nb0 < r_eff) {
+      // weight rows of the four B fragments
+      const uint16_t* wrow[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int j = nb0 + t * 16 + lr;
+        wrow[t] = nullptr;
+        if (j < r_eff) {
+          const int64_t page = seg_page(p.t, base_li + j);
+          if (page >= 0) wrow[t] = wg + page * p.w_stride;
+        }
+      }
+      const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
+      f32x4 acc[2][4];
+#pragma unroll
+      for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+      for (int s = wave; s < ksteps; s += kShrWaves) {
+        const int k = s * 32 + lg * 8;
+        const bool k_ok = k < p.h_in;
+        u32x4 af[2], bf[4];
+#pragma unroll
+        for (int f = 0; f < 2; ++f) af[f] = k_ok ? ldg16(xrow[f] + k) : zero16();
+#pragma unroll
+        for (int t = 0; t < 4; ++t) bf[t] = (k_ok && t < n_tiles && wrow[t] != nullptr) ? ldg16(wrow[t] + k) : zero16();
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          if (t < n_tiles) {
+#pragma unroll
+            for (int f = 0; f < 2; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
+          }
+        }
+      }
+      // C tile: lane holds column lr, rows 4*lg + i
+      float* mine = s_part + wave * (kShrTM * kShrLd);
+#pragma unroll
+      for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[(f * 16 + lg * 4 + i) * kShrLd + t * 16 + lr] = acc[f][t][i];
+    }
+    __syncthreads();
+    for (int idx = tid; idx < kShrTM * kShrNB; idx += kShrThreads) {
+      const int m = idx / kShrNB, c = idx - m * kShrNB;
+      if (m < m_cnt && c < nb_cnt) {
+        float v = 0.f;
+        if (nb0 + c < r_eff) {
+#pragma unroll
+          for (int wv = 0; wv < kShrWaves; ++wv) v += s_part[wv * (kShrTM * kShrLd) + m * kShrLd + c];
+        }
+        og[(int64_t)(row0 + m0 + m) * p.o_stride + nb0 + c] = T::from_float(v);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------
+// expand
+// ---------------------------------------------------------------------------
+struct SegExpandArgs {
+  void* o;
+  const void* x;
+  const void* w;
+  const void* scales;
+  SegTables t;
+  int64_t x_stride, w_stride, o_stride;
+  int64_t page_elems;
+  int scales_dtype;
+  int feat_out, max_rank, qkvo, m_tiles, n_chunks;
+  int vec_ok;
+};
+
+constexpr int kExpThreads = 256;
+constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, each 32 token rows
+constexpr int kExpTMW = 32;                     // token rows per wavefront
+constexpr int kExpTM = kExpTMW * kExpWaves;     // token rows per workgroup
+constexpr int kExpNO = 256;                     // outputs per workgroup
+constexpr int kExpOB = 64;                      // outputs per MFMA block
+
+template <typename T>
+__device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale, int row0,
+                               int m0, int m_cnt, int n0, int n_cnt) {
+  const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* w = reinterpret_cast<const uint16_t*>(p.w);
+  uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
+  const uint32_t page_elems = (uint32_t)p.page_elems;
+  for (int idx = threadIdx.x; idx < m_cnt * n_cnt; idx += kExpThreads) {
+    const int m = idx / n_cnt, n = n0 + (idx - m * n_cnt);
+    const int64_t row = row0 + m0 + m;
+    float acc = 0.f;
+    for (int d = 0; d < r_eff; ++d) {
+      const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
+      const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
+      const int64_t page = seg_page(p.t, base_li + pg);
+      if (page < 0) continue;
+      acc = __builtin_fmaf(T::to_float(x[row * p.x_stride + d]), T::to_float(w[page * p.w_stride + off]), acc);
+    }
+    uint16_t* op = o + row * p.o_stride + n;
+    *op = T::from_float(T::to_float(*op) + acc * scale);
+  }
+}
+
+// KS = number of 32-wide K steps that cover the rank (1, 2 or 4)
+template <typename T, int KS>
+__device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
+                                            int row0, int m0w, int m_cnt_w, int n0, int n_end) {
+  const int lane = threadIdx.x & 63;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
+  uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
+  const uint32_t page_elems = (uint32_t)p.page_elems;
+
+  // B operand: this wavefront's token rows x rank, kept for all output blocks
+  u32x4 bfrag[2][KS];
+  int64_t orow[2];
+  bool row_ok[2];
+#pragma unroll
+  for (int f = 0; f < 2; ++f) {
+    const int m = f * 16 + lr;
+    row_ok[f] = m < m_cnt_w;
+    const int64_t row = row0 + m0w + (row_ok[f] ? m : 0);
+    orow[f] = row * p.o_stride;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int d = s * 32 + lg * 8;
+      bfrag[f][s] = (row_ok[f] && d < r_eff) ? ldg16(xg + row * p.x_stride + d) : zero16();
+    }
+  }
+
+  for (int nb = n0; nb < n_end; nb += kExpOB) {
+    // A operand: MFMA tile t row m <-> output nb + 16*(m/4) + 4*t + (m%4), so that
+    // the four C tiles give every lane 16 consecutive outputs of one token row
+    u32x4 afrag[4][KS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int n = nb + 16 * (lr >> 2) + 4 * t + (lr & 3);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int d = s * 32 + lg * 8;
+        afrag[t][s] = zero16();
+        if (n < p.feat_out && d < r_eff) {
+          const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
+          const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
+          const int64_t page = seg_page(p.t, base_li + pg);
+          if (page >= 0) afrag[t][s] = ldg16(wg + page * p.w_stride + off);
+        }
+      }
+    }
+    const int nl = nb + 16 * lg;  // this lane's 16 outputs start here
+    u32x4 yv[2][2];
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        yv[f][h] = (row_ok[f] && nl + 8 * h < p.feat_out) ? ldg16(og + orow[f] + nl + 8 * h) : zero16();
+
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(afrag[t][s], bfrag[f][s], acc[f][t]);
+      }
+    // C tile t: lane holds token column lr, output rows 4*lg + i  ->  output nl + 4*t + i
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        if (row_ok[f] && nl + 8 * h < p.feat_out) {
+          u32x4 out;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            // elements 8h + 2q, 8h + 2q + 1 of the lane's 16 outputs
+            const int e0 = 8 * h + 2 * q;
+            const float d0 = acc[f][e0 >> 2][e0 & 3] * scale;
+            const float d1 = acc[f][(e0 + 1) >> 2][(e0 + 1) & 3] * scale;
+            const uint16_t lo = T::from_float(T::lo(yv[f][h][q]) + d0);
+            const uint16_t hi = T::from_float(T::hi(yv[f][h][q]) + d1);
+            out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+          }
+          *reinterpret_cast<u32x4*>(og + orow[f] + nl + 8 * h) = out;
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p) {
+  const int wave = threadIdx.x >> 6;
+  int blk = blockIdx.x;
+  const int chunk = blk % p.n_chunks;
+  blk /= p.n_chunks;
+  const int req = blk / p.m_tiles;
+  const int m0 = (blk - req * p.m_tiles) * kExpTM;
+  int64_t a;
+  int r, row0, rows;
+  if (!seg_lookup(p.t, req, a, r, row0, rows)) return;
+  if (m0 >= rows) return;
+  const int r_eff = r < p.max_rank ? r : p.max_rank;
+  if (r_eff <= 0) return;
+  const int m_cnt = rows - m0 < kExpTM ? rows - m0 : kExpTM;
+  const int n0 = chunk * kExpNO;
+  const int n_end = n0 + kExpNO < p.feat_out ? n0 + kExpNO : p.feat_out;
+  const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
+  const float scale = load_scale(p.scales, p.scales_dtype, a);
+  if (!p.vec_ok || (r & 7) != 0 || (r_eff & 7) != 0 || r_eff > 128) {
+    expand_generic<T>(p, r, r_eff, base_li, scale, row0, m0, m_cnt, n0, n_end - n0);
+    return;
+  }
+  const int m0w = m0 + wave * kExpTMW;
+  if (m0w >= rows) return;
+  const int m_cnt_w = rows - m0w < kExpTMW ? rows - m0w : kExpTMW;
+  if (r_eff <= 32)
+    expand_mfma<T, 1>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+  else if (r_eff <= 64)
+    expand_mfma<T, 2>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+  else
+    expand_mfma<T, 4>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+int fill_seg_tables(SegTables& t, const slora_tables* in, const int32_t* b_start_loc, const int32_t* b_seq_len,
+                    const int64_t* b_indicies, int64_t n_requests, int64_t n_tokens, int64_t n_pages) {
+  if (in == nullptr || in->a_start == nullptr || in->a_len == nullptr || in->a_loc == nullptr ||
+      b_start_loc == nullptr || b_seq_len == nullptr || b_indicies == nullptr)
+    return SLORA_ERR_NULL_POINTER;
+  if (in->n_adapters < 0 || in->n_loc < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n_requests > (1 << 24) || n_tokens > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  t.a_start = in->a_start;
+  t.a_len = in->a_len;
+  t.a_loc = in->a_loc;
+  t.b_start_loc = b_start_loc;
+  t.b_seq_len = b_seq_len;
+  t.b_indicies = b_indicies;
+  t.n_adapters = in->n_adapters;
+  t.n_loc = in->n_loc;
+  t.n_pages = n_pages;
+  t.n_requests = (int)n_requests;
+  t.n_tokens = (int)n_tokens;
+  return SLORA_OK;
+}
+
+template <typename T>
+int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
+  const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
+  auto kernel = sgmm_shrink_kernel<T>;
+  static bool attr_done = false;  // benign if two threads race: the call is idempotent
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return SLORA_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles;
+  if (grid <= 0) return SLORA_OK;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+template <typename T>
+int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
+  const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles * p.n_chunks;
+  if (grid <= 0) return SLORA_OK;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(sgmm_expand_kernel<T>, dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+}  // namespace
+}  // namespace slora
+
+extern "C" {
+
+int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables* tables, const int32_t* b_start_loc,
+                      const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
+                      int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride,
+                      int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype, void* stream) {
+  using namespace slora;
+  if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
+  if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || h_in < 0 || max_rank < 0) return SLORA_ERR_BAD_SHAPE;
+  if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
+  if (x_row_stride < h_in || w_row_stride < h_in || o_row_stride < max_rank) return SLORA_ERR_BAD_SHAPE;
+  if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0) return SLORA_OK;
+  SegShrinkArgs p{};
+  int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
+  if (rc != SLORA_OK) return rc;
+  if (o == nullptr || x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (h_in == 0 || h_in > (1 << 21) || max_rank > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
+  p.o = o;
+  p.x = x;
+  p.w = w;
+  p.x_stride = x_row_stride;
+  p.w_stride = w_row_stride;
+  p.o_stride = o_row_stride;
+  p.h_in = (int)h_in;
+  p.max_rank = (int)max_rank;
+  p.qkvo = qkvo;
+  p.m_tiles = (int)((max_input_len + kShrTM - 1) / kShrTM);
+  p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, s) : launch_seg_shrink<BF16>(p, s);
+}
+
+int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables* tables, const void* scales,
+                      int scales_dtype, const int32_t* b_start_loc, const int32_t* b_seq_len,
+                      const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len, int64_t n_tokens,
+                      int64_t feat_out, int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
+                      int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype,
+                      void* stream) {
+  using namespace slora;
+  if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
+  if (scales_dtype != SLORA_DTYPE_F16 && scales_dtype != SLORA_DTYPE_BF16 && scales_dtype != SLORA_DTYPE_F32)
+    return SLORA_ERR_BAD_DTYPE;
+  if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || feat_out < 0 || max_rank < 0 || page_elems < 0)
+    return SLORA_ERR_BAD_SHAPE;
+  if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
+  if (page_elems == 0) page_elems = feat_out;  // the reference's convention: page width == output width
+  if (x_row_stride < max_rank || w_row_stride < page_elems || o_row_stride < feat_out) return SLORA_ERR_BAD_SHAPE;
+  if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0 || feat_out == 0) return SLORA_OK;
+  SegExpandArgs p{};
+  int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
+  if (rc != SLORA_OK) return rc;
+  if (o == nullptr || x == nullptr || w == nullptr || scales == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (feat_out > (1 << 21) || max_rank > SLORA_MAX_RANK || page_elems > (1LL << 30)) return SLORA_ERR_UNSUPPORTED;
+  p.o = o;
+  p.x = x;
+  p.w = w;
+  p.scales = scales;
+  p.scales_dtype = scales_dtype;
+  p.x_stride = x_row_stride;
+  p.w_stride = w_row_stride;
+  p.o_stride = o_row_stride;
+  p.page_elems = page_elems;
+  p.feat_out = (int)feat_out;
+  p.max_rank = (int)max_rank;
+  p.qkvo = qkvo;
+  p.m_tiles = (int)((max_input_len + kExpTM - 1) / kExpTM);
+  p.n_chunks = (int)((feat_out + kExpNO - 1) / kExpNO);
+  p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
+             (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_expand<F16>(p, s) : launch_seg_expand<BF16>(p, s);
+}
+
+}  // extern "C"

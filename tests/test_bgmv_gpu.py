@@ -1,0 +1,304 @@
+"""Decode shrink / expand on the GPU against the CPU oracle.
+
+Everything goes through the C ABI of libslora_hip.so (the Python mirror of
+``dispatch_bgmv`` is a ctypes call).  Tolerance for floating point is the one
+the task states: rtol 1e-2, atol 1e-3 in fp16 and bf16.  Gather/index work is
+checked bit-exactly with integer-valued cases.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import lora_oracle as O
+from lora_cases import make_case
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-2, 1e-3
+TDT = {"f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def dev(a, dtype, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device=device, dtype=dtype)
+
+
+def host(t):
+    return t.detach().to(torch.float32).cpu().numpy()
+
+
+class GpuCase:
+    def __init__(self, c, device, heads=None):
+        tdt = TDT[c.dtype]
+        heads = heads or (4 if c.page_elems % 4 == 0 else 1)
+        self.key = dev(c.key, tdt, device).view(c.n_pages, heads, c.page_elems // heads)
+        self.value = dev(c.value, tdt, device).view(c.n_pages, heads, c.page_elems // heads)
+        self.a_start = dev(c.a_start, torch.int64, device)
+        self.a_len = dev(c.a_len, torch.int64, device)
+        self.a_loc = dev(c.a_loc, torch.int64, device)
+        self.bins = dev(c.bins, torch.int64, device)
+        self.scales = dev(c.scales, torch.float16, device)
+        self.x = dev(c.x, tdt, device)
+        self.tdt = tdt
+
+
+def run_chain(c, g, p, R, device, y0=None):
+    from slora_hip import dispatch_bgmv
+    delta = torch.zeros((c.batch, R), dtype=g.tdt, device=device)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins, p, g.scales)
+    y = torch.zeros((c.batch, c.h_out[p]), dtype=g.tdt, device=device) if y0 is None else dev(y0, g.tdt, device)
+    dispatch_bgmv(y, delta, g.value, g.a_start, g.a_len, g.a_loc, g.bins, p, g.scales)
+    torch.cuda.synchronize()
+    return host(delta), host(y)
+
+
+def oracle_chain(c, p, R, y0=None):
+    delta = O.ref_bgmv_shrink(np.zeros((c.batch, R), np.float32), c.x, c.key, c.a_start, c.a_len, c.a_loc, c.bins, p,
+                              dtype=c.dtype)
+    y0 = np.zeros((c.batch, c.h_out[p]), np.float32) if y0 is None else y0
+    y = O.ref_bgmv_expand(y0, delta, c.value, c.a_start, c.a_len, c.a_loc, c.bins, p, c.scales, dtype=c.dtype)
+    return delta, y
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,ranks,batch", [
+    (256, [8, 16, 32, 64], 37),
+    (1024, [8, 16], 128),          # shape of test_kernel_correctness_multi_rank.py
+    (4096, [64, 32, 16, 8, 64, 8], 64),
+    (5120, [64, 32, 16], 19),
+    (768, [128, 8], 9),
+])
+def test_decode_chain_matches_oracle(gpu, dtype, hidden, ranks, batch):
+    c = make_case(100 + hidden + batch, hidden, ranks, batch, dtype=dtype, zipf_alpha=1.0)
+    g = GpuCase(c, gpu)
+    R = max(ranks)
+    for p in range(4):
+        y0 = O.round_to(np.random.default_rng(p).standard_normal((batch, hidden)).astype(np.float32), dtype)
+        d_gpu, y_gpu = run_chain(c, g, p, R, gpu, y0)
+        d_ref, y_ref = oracle_chain(c, p, R, y0)
+        np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+        # expand is checked on the GPU's own shrink output so one rounding flip in delta is not amplified
+        y_ref2 = O.ref_bgmv_expand(y0, d_gpu, c.value, c.a_start, c.a_len, c.a_loc, c.bins, p, c.scales, dtype=dtype)
+        np.testing.assert_allclose(y_gpu, y_ref2, rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(y_gpu, y_ref, rtol=2 * RTOL, atol=4 * ATOL)
+
+
+def test_reference_kernel_test_shapes(gpu):
+    """The fixture of test/kernel/test_kernel_correctness.py:57-95: H=4096,
+    R=128, N=128, 2 adapters back to back, identity a_loc, scaling 1, qkvo=1,
+    expand; checked against that script's closed form."""
+    rng = np.random.default_rng(42)
+    H, R, N, n_ad, qkvo = 4096, 128, 128, 2, 1
+    key = O.round_to(rng.standard_normal((R * 4 * n_ad, H)).astype(np.float32), "f16")
+    a_len = np.full(n_ad, R * 4, np.int64)
+    a_start = np.array([0, R * 4], np.int64)
+    a_loc = np.arange(R * 4 * n_ad, dtype=np.int64)
+    bins = np.repeat(np.arange(n_ad), N // n_ad).astype(np.int64)
+    x = O.round_to(rng.standard_normal((N, R)).astype(np.float32), "f16")
+    ref = np.zeros((N, H))
+    for i in range(N):
+        a = bins[i]
+        a_w = key[a_start[a] + qkvo * R: a_start[a] + (qkvo + 1) * R].reshape(H, R).T
+        ref[i] = x[i].astype(np.float64) @ a_w.astype(np.float64)
+    from slora_hip import dispatch_bgmv
+    y = torch.zeros((N, H), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(y, dev(x, torch.float16, gpu), dev(key, torch.float16, gpu).view(-1, 32, H // 32),
+                  dev(a_start, torch.int64, gpu), dev(a_len, torch.int64, gpu), dev(a_loc, torch.int64, gpu),
+                  dev(bins, torch.int64, gpu), qkvo, torch.ones(n_ad, dtype=torch.float16, device=gpu))
+    np.testing.assert_allclose(host(y), ref, rtol=RTOL, atol=2e-2)  # |ref| ~ 11, fp16 ulp there is 8e-3
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gather_is_bit_exact(gpu, dtype):
+    """Integer-valued weights and activations: every partial sum is exact in
+    fp32 and the results are exact in the storage type, so equality is
+    bitwise.  Any wrong page / offset / split shows."""
+    rng = np.random.default_rng(7)
+    H, ranks, batch = 512, [8, 16, 32, 8, 64], 96
+    c = make_case(7, H, ranks, batch, dtype=dtype, zipf_alpha=0.8)
+    for i, r in enumerate(ranks):
+        c.A[i] = [rng.integers(-2, 3, (H, r)).astype(np.float32) for _ in range(4)]
+        c.B[i] = [rng.integers(-2, 3, (r, H)).astype(np.float32) for _ in range(4)]
+        loc = c.a_loc[c.a_start[i]: c.a_start[i] + 4 * r]
+        O.load_into_pool(c.key, c.value, O.pack_w_combined(c.A[i], c.B[i], H), loc)
+    # sparse small-integer activations keep |delta| and |y| small enough to be exact in bf16 too
+    x = np.zeros((batch, H), np.float32)
+    for t in range(batch):
+        idx = rng.choice(H, size=3, replace=False)
+        x[t, idx] = rng.integers(-2, 3, 3)
+    c.x = x
+    c.scales = np.array([1.0, 2.0, 0.5, 1.0, 0.25], np.float32)
+    g = GpuCase(c, gpu)
+    for p in range(4):
+        d_gpu, y_gpu = run_chain(c, g, p, 64, gpu)
+        for t in range(batch):
+            a = c.bins[t]
+            d = c.x[t] @ c.A[a][p]
+            assert np.array_equal(d_gpu[t, : ranks[a]], d), (p, t)
+            assert np.all(d_gpu[t, ranks[a]:] == 0)
+            want = O.round_to((d @ c.B[a][p]) * c.scales[a], dtype)
+            assert np.array_equal(y_gpu[t], want), (p, t)
+
+
+def test_shrink_leaves_columns_beyond_rank_untouched(gpu):
+    c = make_case(8, 256, [8, 16], 20, dtype="f16")
+    g = GpuCase(c, gpu)
+    from slora_hip import dispatch_bgmv
+    delta = torch.full((c.batch, 32), 3.0, dtype=torch.float16, device=gpu)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins, 2, g.scales)
+    d = host(delta)
+    for t in range(c.batch):
+        r = c.ranks[c.bins[t]]
+        assert np.all(d[t, r:] == 3.0)
+        assert not np.any(d[t, :r] == 3.0)
+
+
+def test_expand_ignores_garbage_beyond_rank_and_scale_zero(gpu):
+    c = make_case(9, 256, [8, 16, 32], 33, dtype="f16")
+    g = GpuCase(c, gpu)
+    from slora_hip import dispatch_bgmv
+    R = 32
+    delta = torch.zeros((c.batch, R), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins, 1, g.scales)
+    y1 = torch.zeros((c.batch, 256), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(y1, delta, g.value, g.a_start, g.a_len, g.a_loc, g.bins, 1, g.scales)
+    junk = delta.clone()
+    for t in range(c.batch):
+        junk[t, c.ranks[c.bins[t]]:] = 1000.0
+    y2 = torch.zeros_like(y1)
+    dispatch_bgmv(y2, junk, g.value, g.a_start, g.a_len, g.a_loc, g.bins, 1, g.scales)
+    assert torch.equal(y1, y2)
+    y3 = torch.randn_like(y1)
+    y3_before = y3.clone()
+    dispatch_bgmv(y3, delta, g.value, g.a_start, g.a_len, g.a_loc, g.bins, 1, torch.zeros_like(g.scales))
+    assert torch.equal(y3, y3_before)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gqa_narrow_kv_and_wide_pages(gpu, dtype):
+    """Output narrower than a page (k/v of grouped-query attention): hidden
+    1024, k/v width 256, page = 1024 elements."""
+    c = make_case(11, 1024, [64, 16, 8], 40, dtype=dtype, h_out=[1024, 256, 256, 1024])
+    g = GpuCase(c, gpu)
+    for p in range(4):
+        d_gpu, y_gpu = run_chain(c, g, p, 64, gpu)
+        y_ref = O.ref_bgmv_expand(np.zeros((c.batch, c.h_out[p]), np.float32), d_gpu, c.value, c.a_start, c.a_len,
+                                  c.a_loc, c.bins, p, c.scales, dtype=dtype)
+        np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_odd_rank_and_rank_above_columns(gpu):
+    """Ranks that are not a multiple of 8 take the element-wise path; an
+    adapter whose rank exceeds the delta width uses only the columns there are."""
+    c = make_case(12, 256, [4, 12, 8, 24], 30, dtype="f16")
+    g = GpuCase(c, gpu)
+    for p in (0, 3):
+        for R in (24, 16):
+            d_gpu, y_gpu = run_chain(c, g, p, R, gpu)
+            d_ref, _ = oracle_chain(c, p, R)
+            np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+            y_ref = O.ref_bgmv_expand(np.zeros((c.batch, 256), np.float32), d_gpu, c.value, c.a_start, c.a_len,
+                                      c.a_loc, c.bins, p, c.scales, dtype="f16")
+            np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("batch", [1, 7, 513, 1500])
+def test_ragged_batches_and_popular_adapter(gpu, batch):
+    """Batches that do not fill a workgroup group, batches longer than one
+    scan chunk, and one adapter owning most tokens (long runs)."""
+    bins = np.random.default_rng(batch).choice(4, size=batch, p=[0.85, 0.05, 0.05, 0.05])
+    c = make_case(13 + batch, 512, [16, 8, 64, 32], batch, dtype="f16", bins=bins)
+    g = GpuCase(c, gpu)
+    d_gpu, y_gpu = run_chain(c, g, 0, 64, gpu)
+    d_ref, _ = oracle_chain(c, 0, 64)
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+    y_ref = O.ref_bgmv_expand(np.zeros((batch, 512), np.float32), d_gpu, c.value, c.a_start, c.a_len, c.a_loc,
+                              c.bins, 0, c.scales, dtype="f16")
+    np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_empty_batch_and_zero_rank(gpu):
+    from slora_hip import dispatch_bgmv
+    c = make_case(14, 256, [8, 0, 16], 12, dtype="f16", bins=np.array([0, 1, 2] * 4))
+    g = GpuCase(c, gpu)
+    d_gpu, y_gpu = run_chain(c, g, 0, 16, gpu)
+    assert np.all(d_gpu[1::3] == 0) and np.all(y_gpu[1::3] == 0)  # rank-0 adapter: nothing happens
+    d_ref, _ = oracle_chain(c, 0, 16)
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+    e = torch.zeros((0, 256), dtype=torch.float16, device=gpu)
+    d = torch.zeros((0, 16), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(d, e, g.key, g.a_start, g.a_len, g.a_loc, g.bins[:0], 0, g.scales)
+    dispatch_bgmv(e, d, g.value, g.a_start, g.a_len, g.a_loc, g.bins[:0], 0, g.scales)
+    torch.cuda.synchronize()
+
+
+def test_out_of_range_indices_are_skipped_not_faulted(gpu):
+    """Adapter ids or page ids outside the tables: the token / row is skipped."""
+    from slora_hip import dispatch_bgmv
+    c = make_case(15, 256, [8, 16], 8, dtype="f16", bins=np.array([0, 1, 0, 1, 0, 1, 0, 1]))
+    g = GpuCase(c, gpu)
+    bad_bins = g.bins.clone()
+    bad_bins[3] = 99
+    bad_bins[4] = -1
+    delta = torch.full((8, 16), 5.0, dtype=torch.float16, device=gpu)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, g.a_loc, bad_bins, 0, g.scales)
+    d = host(delta)
+    assert np.all(d[3] == 5.0) and np.all(d[4] == 5.0)
+    bad_loc = g.a_loc.clone()
+    bad_loc[0] = c.n_pages + 5  # adapter 0, projection q, row 0
+    delta.fill_(5.0)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, bad_loc, g.bins, 0, g.scales)
+    d = host(delta)
+    assert np.all(d[0::2, 0] == 5.0)
+    d_ref, _ = oracle_chain(c, 0, 16)
+    np.testing.assert_allclose(d[0::2, 1:8], d_ref[0::2, 1:8], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_fused_qkv_equals_three_calls(gpu, dtype):
+    from slora_hip import dispatch_bgmv, dispatch_bgmv_qkv_shrink, dispatch_bgmv_qkv_expand
+    c = make_case(16, 1024, [64, 8, 32, 16], 70, dtype=dtype, h_out=[1024, 256, 256, 1024], zipf_alpha=1.0)
+    g = GpuCase(c, gpu)
+    R = 64
+    sep = [torch.zeros((c.batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+    fus = [torch.zeros((c.batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+    for p in range(3):
+        dispatch_bgmv(sep[p], g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins, p, g.scales)
+    dispatch_bgmv_qkv_shrink(fus[0], fus[1], fus[2], g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins)
+    for p in range(3):
+        assert torch.equal(sep[p], fus[p])
+    y0 = [torch.randn((c.batch, c.h_out[p]), dtype=g.tdt, device=gpu) for p in range(3)]
+    ys = [t.clone() for t in y0]
+    yf = [t.clone() for t in y0]
+    for p in range(3):
+        dispatch_bgmv(ys[p], sep[p], g.value, g.a_start, g.a_len, g.a_loc, g.bins, p, g.scales)
+    dispatch_bgmv_qkv_expand(yf[0], yf[1], yf[2], fus[0], fus[1], fus[2], g.value, g.a_start, g.a_len, g.a_loc,
+                             g.bins, g.scales)
+    for p in range(3):
+        assert torch.equal(ys[p], yf[p])
+
+
+def test_scaling_table_read_in_its_own_dtype(gpu):
+    """bf16 activations with the fp16 scaling table the reference keeps
+    (infer_adapter.py:33): the table must be read as fp16."""
+    c = make_case(17, 256, [8, 16], 10, dtype="bf16")
+    g = GpuCase(c, gpu)
+    d_gpu, y_gpu = run_chain(c, g, 0, 16, gpu)
+    y_ref = O.ref_bgmv_expand(np.zeros((10, 256), np.float32), d_gpu, c.value, c.a_start, c.a_len, c.a_loc, c.bins, 0,
+                              c.scales, dtype="bf16")
+    np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_denormal_weights_are_not_flushed(gpu):
+    """The reference's dummy adapters are U(-1e-3, 1e-3) (lora_layer_weight.py:41-56):
+    a good part of such weights is subnormal in fp16 and must still count."""
+    c = make_case(18, 1024, [8, 16], 16, dtype="f16")
+    rng = np.random.default_rng(18)
+    for i, r in enumerate(c.ranks):
+        c.A[i] = [O.round_to(rng.uniform(-6e-5, 6e-5, (1024, r)).astype(np.float32), "f16") for _ in range(4)]
+        loc = c.a_loc[c.a_start[i]: c.a_start[i] + 4 * r]
+        O.load_into_pool(c.key, c.value, O.pack_w_combined(c.A[i], c.B[i], 1024), loc)
+    c.x = O.round_to(np.abs(c.x) * 8, "f16")
+    g = GpuCase(c, gpu)
+    d_gpu, _ = run_chain(c, g, 0, 16, gpu)
+    d_ref, _ = oracle_chain(c, 0, 16)
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=1e-5)

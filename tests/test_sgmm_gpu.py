@@ -1,0 +1,162 @@
+"""Prefill segmented shrink / expand on the GPU against the CPU oracle, through
+the C ABI.  Tolerance: rtol 1e-2, atol 1e-3 (fp16 and bf16)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import lora_oracle as O
+from lora_cases import make_case, make_segments
+from test_bgmv_gpu import GpuCase, dev, host, RTOL, ATOL, TDT
+
+pytestmark = pytest.mark.gpu
+
+
+def seg_case(seed, hidden, ranks, n_req, lo, hi, dtype, h_out=None, sort=True):
+    start, lens, ids = make_segments(seed, n_req, lo, hi, len(ranks), sort_by_adapter=sort)
+    T = int(lens.sum())
+    c = make_case(seed, hidden, ranks, batch=T, dtype=dtype, bins=np.repeat(ids, lens), h_out=h_out)
+    c.start, c.lens, c.ids = start, lens, ids
+    return c
+
+
+def run_prefill(c, g, p, R, device, o0, y0):
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand
+    start = dev(c.start, torch.int32, device)
+    lens = dev(c.lens, torch.int32, device)
+    ids = dev(c.ids, torch.int64, device)
+    max_len = int(c.lens.max()) if len(c.lens) else 0
+    delta = dev(o0, g.tdt, device)
+    w_a = g.key.view(c.n_pages, c.page_elems)
+    w_b = g.value.view(c.n_pages, c.page_elems)
+    lora_get_qkvo_fwd_shrink(g.x, w_a, delta, g.a_loc, g.a_start, g.a_len, start, lens, ids, c.hidden, p, R, max_len)
+    y = dev(y0, g.tdt, device)
+    lora_get_qkvo_fwd_expand(delta, w_b, y, g.scales, g.a_loc, g.a_start, g.a_len, start, lens, ids, c.h_out[p], p, R,
+                             max_len)
+    torch.cuda.synchronize()
+    return host(delta), host(y)
+
+
+def check(c, g, p, R, device, seed=0):
+    rng = np.random.default_rng(seed)
+    T = c.batch
+    o0 = O.round_to(rng.standard_normal((T, R)).astype(np.float32), c.dtype)  # garbage that must be overwritten
+    y0 = O.round_to(rng.standard_normal((T, c.h_out[p])).astype(np.float32), c.dtype)
+    d_gpu, y_gpu = run_prefill(c, g, p, R, device, o0, y0)
+    d_ref = O.ref_prefill_shrink(o0, c.x, c.key, c.a_loc, c.a_start, c.a_len, c.start, c.lens, c.ids, p, R, c.dtype)
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+    y_ref = O.ref_prefill_expand(y0, d_gpu, c.value, c.scales, c.a_loc, c.a_start, c.a_len, c.start, c.lens, c.ids, p,
+                                 R, c.dtype)
+    np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+    return d_gpu, y_gpu
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,ranks,n_req,lo,hi", [
+    (256, [8, 16, 32, 64], 9, 1, 70),
+    (1024, [64, 8, 16], 6, 8, 200),
+    (4096, [64, 32, 16, 8], 8, 8, 300),
+    (5120, [64, 32, 16], 4, 100, 256),
+    (512, [128, 8], 5, 1, 40),
+])
+def test_prefill_chain_matches_oracle(gpu, dtype, hidden, ranks, n_req, lo, hi):
+    c = seg_case(200 + hidden + n_req, hidden, ranks, n_req, lo, hi, dtype)
+    g = GpuCase(c, gpu)
+    R = max(ranks)
+    for p in range(4):
+        check(c, g, p, R, gpu, seed=p)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_prefill_gather_bit_exact(gpu, dtype):
+    rng = np.random.default_rng(5)
+    H, ranks = 256, [8, 16, 32, 64]
+    c = seg_case(5, H, ranks, 7, 1, 50, dtype, sort=False)
+    for i, r in enumerate(ranks):
+        c.A[i] = [rng.integers(-2, 3, (H, r)).astype(np.float32) for _ in range(4)]
+        c.B[i] = [rng.integers(-2, 3, (r, H)).astype(np.float32) for _ in range(4)]
+        loc = c.a_loc[c.a_start[i]: c.a_start[i] + 4 * r]
+        O.load_into_pool(c.key, c.value, O.pack_w_combined(c.A[i], c.B[i], H), loc)
+    x = np.zeros((c.batch, H), np.float32)
+    for t in range(c.batch):
+        idx = rng.choice(H, size=3, replace=False)
+        x[t, idx] = rng.integers(-2, 3, 3)
+    c.x = x
+    c.scales = np.array([1.0, 2.0, 0.5, 0.25], np.float32)
+    g = GpuCase(c, gpu)
+    for p in range(4):
+        o0 = np.full((c.batch, 64), 9.0, np.float32)
+        y0 = np.zeros((c.batch, H), np.float32)
+        d_gpu, y_gpu = run_prefill(c, g, p, 64, gpu, o0, y0)
+        for t in range(c.batch):
+            a = c.bins[t]
+            d = c.x[t] @ c.A[a][p]
+            assert np.array_equal(d_gpu[t, : ranks[a]], d), (p, t)
+            assert np.all(d_gpu[t, ranks[a]:] == 0), (p, t)      # zero fill up to max_rank
+            assert np.array_equal(y_gpu[t], O.round_to((d @ c.B[a][p]) * c.scales[a], dtype)), (p, t)
+
+
+def test_prefill_unowned_rows_and_empty_requests(gpu):
+    """Rows no request owns stay as they were; zero-length requests do nothing."""
+    c = make_case(6, 256, [8, 16], batch=40, dtype="f16", bins=np.zeros(40, np.int64))
+    c.start = np.array([3, 20, 30], np.int32)
+    c.lens = np.array([5, 0, 7], np.int32)
+    c.ids = np.array([1, 0, 0], np.int64)
+    c.bins[3:8] = 1
+    g = GpuCase(c, gpu)
+    o0 = np.full((40, 16), 5.0, np.float32)
+    y0 = np.full((40, 256), 2.0, np.float32)
+    d_gpu, y_gpu = run_prefill(c, g, 1, 16, gpu, o0, y0)
+    owned = np.zeros(40, bool)
+    owned[3:8] = True
+    owned[30:37] = True
+    assert np.all(d_gpu[~owned] == 5.0) and np.all(y_gpu[~owned] == 2.0)
+    d_ref = O.ref_prefill_shrink(o0, c.x, c.key, c.a_loc, c.a_start, c.a_len, c.start, c.lens, c.ids, 1, 16, "f16")
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_prefill_strided_views_and_odd_layouts(gpu):
+    """x / o as row-strided views (the reference passes strides), a rank that
+    is not a multiple of 8 and an output width that is not a multiple of 8
+    (element-wise path)."""
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand
+    c = seg_case(7, 256, [12, 8, 20], 5, 3, 40, "f16")
+    g = GpuCase(c, gpu)
+    R = 24
+    T = c.batch
+    start, lens, ids = dev(c.start, torch.int32, gpu), dev(c.lens, torch.int32, gpu), dev(c.ids, torch.int64, gpu)
+    max_len = int(c.lens.max())
+    x_wide = torch.zeros((T, 256 + 24), dtype=torch.float16, device=gpu)
+    x_wide[:, :256] = g.x
+    xv = x_wide[:, :256]
+    d_wide = torch.zeros((T, R + 3), dtype=torch.float16, device=gpu)
+    dv = d_wide[:, :R]
+    lora_get_qkvo_fwd_shrink(xv, g.key.view(c.n_pages, 256), dv, g.a_loc, g.a_start, g.a_len, start, lens, ids, 256, 2,
+                             R, max_len)
+    d_ref = O.ref_prefill_shrink(np.zeros((T, R), np.float32), c.x, c.key, c.a_loc, c.a_start, c.a_len, c.start,
+                                 c.lens, c.ids, 2, R, "f16")
+    np.testing.assert_allclose(host(dv), d_ref, rtol=RTOL, atol=ATOL)
+    assert torch.all(d_wide[:, R:] == 0)
+    y_wide = torch.ones((T, 256 + 5), dtype=torch.float16, device=gpu)
+    yv = y_wide[:, :256]
+    lora_get_qkvo_fwd_expand(dv, g.value.view(c.n_pages, 256), yv, g.scales, g.a_loc, g.a_start, g.a_len, start, lens,
+                             ids, 256, 2, R, max_len)
+    y_ref = O.ref_prefill_expand(np.ones((T, 256), np.float32), host(dv), c.value, c.scales, c.a_loc, c.a_start,
+                                 c.a_len, c.start, c.lens, c.ids, 2, R, "f16")
+    np.testing.assert_allclose(host(yv), y_ref, rtol=RTOL, atol=ATOL)
+    assert torch.all(y_wide[:, 256:] == 1)
+
+
+def test_prefill_matches_decode_kernels(gpu):
+    """The two operator families must agree where the reference treats them as
+    interchangeable (lora_unordered_batch_infer.py:334-355)."""
+    from slora_hip import dispatch_bgmv
+    c = seg_case(8, 1024, [64, 16, 32], 6, 5, 90, "f16")
+    g = GpuCase(c, gpu)
+    R = 64
+    d_gpu, y_gpu = run_prefill(c, g, 0, R, gpu, np.zeros((c.batch, R), np.float32), np.zeros((c.batch, 1024), np.float32))
+    delta = torch.zeros((c.batch, R), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(delta, g.x, g.key, g.a_start, g.a_len, g.a_loc, g.bins, 0, g.scales)
+    y = torch.zeros((c.batch, 1024), dtype=torch.float16, device=gpu)
+    dispatch_bgmv(y, delta, g.value, g.a_start, g.a_len, g.a_loc, g.bins, 0, g.scales)
+    np.testing.assert_allclose(host(delta), d_gpu, rtol=RTOL, atol=ATOL)
+    np.testing.assert_allclose(host(y), y_gpu, rtol=2 * RTOL, atol=4 * ATOL)
