@@ -1,0 +1,323 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-LoRA batching hot path on one MI355X.
+
+A "step" is one decode step's LoRA work at the S2 shape: for each of 32 layers,
+q/k/v/o shrink and expand over the same batch of 256 tokens (200 adapters,
+ranks {64,32,16,8}, Zipf(1) adapter popularity), reading adapter pages straight
+from the per-layer unified pool.  The base-model matmuls are not part of it.
+Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line: LoRA tokens/s for the whole step, the roofline figure of
+the dominant kernel (algorithmic bytes per launch / measured launch duration)
+and the reference's torch bmm path timed on this box's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "s-lora_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+METRIC = "LoRA tokens/s + achieved HBM GB/s (% peak), S2 decode BGMV batch 256"
+HBM_PEAK_GBS = 8000.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--batch", type=int, default=256)
+    ap.add_argument("--workload", choices=["s2", "s4", "s6"], default="s2")
+    ap.add_argument("--mode", choices=["dropin", "fused"], default="dropin",
+                    help="dropin: 8 dispatch_bgmv calls per layer as the reference issues them; "
+                         "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer)")
+    ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
+                    help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-reps", type=int, default=0, help="0 = as many as fit in about 15 s")
+    ap.add_argument("--check", action="store_true", help="verify layer 0 against the oracle before timing")
+    return ap.parse_args()
+
+
+class StepBuffers:
+    """Activations and outputs of every layer, distinct per layer so that no
+    call finds its operands cached by the previous layer."""
+
+    def __init__(self, w, device):
+        import torch
+        g = torch.Generator(device=device)
+        g.manual_seed(123)
+        B, H = w.batch, w.hidden
+        self.x_in = [torch.randn((B, H), generator=g, device=device, dtype=torch.float32).to(w.dtype)
+                     for _ in range(w.n_layers)]
+        self.x_att = [torch.randn((B, H), generator=g, device=device, dtype=torch.float32).to(w.dtype)
+                      for _ in range(w.n_layers)]
+        self.y = [[torch.zeros((B, h), device=device, dtype=w.dtype) for h in w.h_out] for _ in range(w.n_layers)]
+        self.delta = [torch.zeros((B, w.max_rank), device=device, dtype=w.dtype) for _ in range(3)]
+
+
+def make_step(w, bufs, mode):
+    import slora_hip
+    bgmv = slora_hip.dispatch_bgmv
+    t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
+
+    def shrink_sweep():
+        for l in range(w.n_layers):
+            for p in range(3):
+                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling)
+            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
+
+    def expand_sweep():
+        for l in range(w.n_layers):
+            for p in range(3):
+                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling)
+            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
+
+    def step_dropin():
+        # call order of lora_unordered_batch_infer.py:254-318, 428-448
+        for l in range(w.n_layers):
+            for p in range(3):
+                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling)
+                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling)
+            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
+            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
+
+    def step_fused():
+        for l in range(w.n_layers):
+            slora_hip.dispatch_bgmv_qkv_shrink(bufs.delta[0], bufs.delta[1], bufs.delta[2], bufs.x_in[l],
+                                               w.key_buffer[l], *t)
+            slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
+                                               bufs.delta[2], w.value_buffer[l], *t, w.a_scaling)
+            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
+            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
+
+    return (step_fused if mode == "fused" else step_dropin), shrink_sweep, expand_sweep
+
+
+def graphed(fn, torch):
+    """Capture fn once on a side stream and return a replay callable."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g.replay
+
+
+def time_region(fn, reps, warmup, torch):
+    """HIP events on the stream the kernels are enqueued on; returns ms per rep."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def check_layer0(w, bufs, torch):
+    """Layer 0, all four projections, every token, against the oracle (the
+    adapter pages of layer 0 are copied to the host for it)."""
+    import numpy as np
+    import slora_hip
+    from oracle import lora_oracle as O
+    dt = "f16" if w.dtype == torch.float16 else "bf16"
+    used = np.unique(w.a_loc_np)
+    remap = np.full(w.n_pages, -1, dtype=np.int64)
+    remap[used] = np.arange(used.size)
+    idx = torch.from_numpy(used).to(w.key_buffer[0].device)
+    key = w.key_buffer[0][idx].reshape(used.size, -1).float().cpu().numpy()
+    val = w.value_buffer[0][idx].reshape(used.size, -1).float().cpu().numpy()
+    loc = remap[w.a_loc_np]
+    t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
+    for p in range(4):
+        x = bufs.x_in[0] if p < 3 else bufs.x_att[0]
+        delta = torch.zeros_like(bufs.delta[0])
+        y = torch.zeros_like(bufs.y[0][p])
+        slora_hip.dispatch_bgmv(delta, x, w.key_buffer[0], *t, p, w.a_scaling)
+        slora_hip.dispatch_bgmv(y, delta, w.value_buffer[0], *t, p, w.a_scaling)
+        torch.cuda.synchronize()
+        d_gpu = delta.float().cpu().numpy()
+        d_ref = O.ref_bgmv_shrink(np.zeros_like(d_gpu), x.float().cpu().numpy(), key, w.a_start_np, w.a_len_np, loc,
+                                  w.bins_np, p, dt)
+        np.testing.assert_allclose(d_gpu, d_ref, rtol=1e-2, atol=1e-3)
+        y_ref = O.ref_bgmv_expand(np.zeros((w.batch, w.h_out[p]), np.float32), d_gpu, val, w.a_start_np, w.a_len_np,
+                                  loc, w.bins_np, p, w.a_scaling.float().cpu().numpy(), dt)
+        np.testing.assert_allclose(y.float().cpu().numpy(), y_ref, rtol=1e-2, atol=1e-3)
+
+
+def cpu_baseline(w, bufs, torch, reps_arg):
+    """The reference's bmm path (gather, zero-padded bmm, scatter-add) in torch
+    float32 on this box's host cores, on ONE layer of the same workload."""
+    import numpy as np
+    from oracle import lora_oracle as O
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    u = w.distinct_adapters()
+    dev = w.key_buffer[0].device
+    A, B, scal = [], [], []
+    for a in u:
+        r = int(w.ranks[a])
+        loc = w.a_loc_np[w.a_start_np[a]: w.a_start_np[a] + 4 * r]
+        idx = torch.from_numpy(loc).to(dev)
+        kp = w.key_buffer[0][idx].reshape(4 * r, -1).float().cpu().numpy()
+        vp = w.value_buffer[0][idx].reshape(4 * r, -1).float().cpu().numpy()
+        a_p, b_p = O.unpack_from_pool(kp, vp, np.arange(4 * r), w.hidden, w.h_out)
+        A.append(a_p)
+        B.append(b_p)
+        scal.append(float(w.scales_np[a]))
+    remap = {int(a): i for i, a in enumerate(u)}
+    bins = np.array([remap[int(b)] for b in w.bins_np])
+    layer = O.BmmCpuLayer(A, B, scal, bins, threads=threads)
+    x_in = bufs.x_in[0].float().cpu()
+    x_att = bufs.x_att[0].float().cpu()
+    ys = [torch.zeros((w.batch, h), dtype=torch.float32) for h in w.h_out]
+    layer.decode(x_in, x_att, ys)  # warm-up
+    t0 = time.perf_counter()
+    layer.decode(x_in, x_att, ys)
+    one = time.perf_counter() - t0
+    reps = reps_arg or max(3, min(30, int(15.0 / max(one, 1e-3))))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        layer.decode(x_in, x_att, ys)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {
+        "value": round(w.batch / (med * w.n_layers), 1),
+        "unit": "tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"1 of {w.n_layers} layers (q/k/v/o gather + padded torch.bmm o bmm + scatter-add, fp32, "
+                  f"{u.size} adapters in batch), median of {reps} reps = {med * 1e3:.1f} ms/layer; "
+                  f"step time extrapolated x{w.n_layers}",
+        "gbps_algorithmic": round(w.layer_bytes() / med / 1e9, 2),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the LoRA path has no cross-GPU part); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    import slora_hip
+    from slora_hip import workloads
+    slora_hip.load_library()
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    if args.workload == "s2":
+        w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch)
+    elif args.workload == "s4":
+        w = workloads.s4_decode(device, n_layers=args.layers, batch=args.batch if args.batch != 256 else 512)
+    else:
+        w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024)
+    bufs = StepBuffers(w, device)
+    step, shrink_sweep, expand_sweep = make_step(w, bufs, args.mode)
+    if args.check:
+        check_layer0(w, bufs, torch)
+
+    run_step, run_shrink, run_expand = step, shrink_sweep, expand_sweep
+    if args.launch == "graph":
+        run_step, run_shrink, run_expand = graphed(step, torch), graphed(shrink_sweep, torch), graphed(expand_sweep, torch)
+
+    # ---- the timed region: exactly K steps between two synchronisations ---------------
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        run_step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    ms_per_step = max(ms_per_step, wall_ms) if args.launch == "direct" else ms_per_step
+
+    # ---- per-kernel launch duration: sweeps of one kernel family, same stream ---------
+    n_launch = w.n_layers * 4
+    reps = max(5, args.steps // 2)
+    shrink_us = time_region(run_shrink, reps, 3, torch) * 1e3 / n_launch
+    expand_us = time_region(run_expand, reps, 3, torch) * 1e3 / n_launch
+    shrink_bytes = sum(w.shrink_bytes() for _ in range(4)) / 4
+    expand_bytes = sum(w.expand_bytes(h) for h in w.h_out) / 4
+    shrink_gbs = shrink_bytes / (shrink_us * 1e-6) / 1e9
+    expand_gbs = expand_bytes / (expand_us * 1e-6) / 1e9
+    dominant = ("bgmv_expand_kernel", expand_us, expand_bytes, expand_gbs) if expand_us >= shrink_us else \
+               ("bgmv_shrink_kernel", shrink_us, shrink_bytes, shrink_gbs)
+
+    step_gbs = w.step_bytes() / (ms_per_step * 1e-3) / 1e9
+    out = {
+        "metric": METRIC,
+        "value": round(w.batch / (ms_per_step * 1e-3), 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16" if w.dtype == torch.float16 else "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "layers": w.n_layers,
+            "batch": w.batch,
+            "distinct_adapters_in_batch": int(w.distinct_adapters().size),
+            "pool_pages_per_layer": w.n_pages,
+            "mode": args.mode,
+            "launch": args.launch,
+            "launches_per_step": w.n_layers * (8 if args.mode == "dropin" else 4),
+        },
+        "step_hbm": {
+            "algorithmic_bytes_per_step": w.step_bytes(),
+            "achieved_GBps": round(step_gbs, 1),
+            "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
+        },
+        "roofline": {
+            "kernel": dominant[0],
+            "bound": "hbm",
+            "achieved": round(dominant[3], 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(dominant[3] / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_launch": int(dominant[2]),
+            "us_per_launch": round(dominant[1], 3),
+        },
+        "kernels": {
+            "bgmv_shrink_kernel": {"us_per_launch": round(shrink_us, 3), "bytes_per_launch": int(shrink_bytes),
+                                   "GBps": round(shrink_gbs, 1), "frac": round(shrink_gbs / HBM_PEAK_GBS, 4)},
+            "bgmv_expand_kernel": {"us_per_launch": round(expand_us, 3), "bytes_per_launch": int(expand_bytes),
+                                   "GBps": round(expand_gbs, 1), "frac": round(expand_gbs / HBM_PEAK_GBS, 4)},
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w, bufs, torch, args.cpu_reps)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

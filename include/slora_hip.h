@@ -110,6 +110,52 @@ SLORA_API int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void*
                           int64_t h_out_v, int64_t page_elems, int64_t n_pages, int dtype,
                           void* stream);
 
+/* ---- per-batch plan (no counterpart in the reference) ----------------------
+ * The reference rebuilds nothing per call because it launches one block per
+ * (token, rank row) and lets most of them exit; here a call walks
+ * bins -> a_len/a_start -> a_loc before it can touch a weight.  Those tables do
+ * not change between the 8 x n_layers calls of one decode step
+ * (lora_unordered_batch_infer.py:254-318 passes the same req_bins and
+ * infer_adapter tables to every call), so a caller may build a plan once per
+ * step and pass it to the *_planned entry points, which then reach the weights
+ * in one table read.  The plan lists the batch's work items: a "run" (up to 4
+ * tokens that share an adapter) times a block of 8 rows, with the tokens and
+ * the page ids of those rows for q, k, v and o.  It is valid as long as bins and the adapter tables keep their
+ * contents.  rank_cap bounds the ranks whose page ids are stored (larger ranks
+ * still work through a_loc).  Results are identical to the stateless calls. */
+
+/* Bytes a plan for `batch` tokens needs (negative: SLORA_ERR_*). */
+SLORA_API int64_t slora_bgmv_plan_bytes(int64_t batch, int64_t rank_cap);
+
+/* Enqueue the plan build on `stream`.  `plan` is a 16-byte aligned device
+ * buffer of at least slora_bgmv_plan_bytes(batch, rank_cap) bytes.  Word 1 of
+ * the finished plan (int32) is the number of items, word 2 the largest rank in
+ * the batch, word 6 the number of runs; a caller may read word 1 back and pass
+ * it as n_items so that a launch has exactly one workgroup per item. */
+SLORA_API int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables,
+                                    const int64_t* bins, int64_t batch, int64_t rank_cap,
+                                    int64_t n_pages, void* stream);
+
+/* slora_bgmv_shrink / slora_bgmv_shrink_qkv with a plan.  nproj = 1: y0 and
+ * qkvo as in slora_bgmv_shrink; nproj = 3: y0,y1,y2 = q,k,v and qkvo = 0.
+ * n_items = 0 launches for the plan's capacity (always enough); a caller that
+ * read the item count back passes it. */
+SLORA_API int slora_bgmv_shrink_planned(const void* plan, int64_t rank_cap, int64_t n_items, int nproj,
+                                        void* y0, void* y1, void* y2, const void* x, const void* w,
+                                        const slora_tables* tables, const int64_t* bins,
+                                        int64_t batch, int64_t h_in, int64_t y_cols,
+                                        int64_t page_elems, int64_t n_pages, int qkvo, int dtype,
+                                        void* stream);
+
+/* slora_bgmv_expand / slora_bgmv_expand_qkv with a plan. */
+SLORA_API int slora_bgmv_expand_planned(const void* plan, int64_t rank_cap, int64_t n_items, int nproj,
+                                        void* y0, void* y1, void* y2, const void* x0, const void* x1,
+                                        const void* x2, const void* w, const slora_tables* tables,
+                                        const int64_t* bins, const void* scales, int scales_dtype,
+                                        int64_t batch, int64_t x_cols, int64_t h_out0,
+                                        int64_t h_out1, int64_t h_out2, int64_t page_elems,
+                                        int64_t n_pages, int qkvo, int dtype, void* stream);
+
 /* Prefill (segmented) shrink.  Replaces lora_get_qkvo_fwd_shrink + _shrink_fwd_kernel
  * (slora/models/peft/triton_kernel/lora/lora_prefill.py:139-164, 57-102).
  * Request i owns token rows b_start_loc[i] + [0, b_seq_len[i]) and uses

@@ -326,3 +326,55 @@ def ref_var_len_copy(old_a_start, old_a_len, old_a_loc, new_a_start, new_size: i
         n = int(old_a_len[i])
         out[int(new_a_start[i]): int(new_a_start[i]) + n] = old_a_loc[int(old_a_start[i]): int(old_a_start[i]) + n]
     return out
+
+
+# ----------------------------------------------------------------------------
+# the reference's torch path on host cores (CPU baseline of the benchmark)
+# ----------------------------------------------------------------------------
+class BmmCpuLayer:
+    """One layer of LoraBmmInfer on the CPU in torch float32: the padded
+    ``batch_lora_A [4, n, H, max_r]`` / ``batch_lora_B [4, n, max_r, H_out]``
+    are built once (lora_bmm_infer.py:33-50); ``decode`` is
+    ``_batch_lora_get_qkv`` + ``_batch_lora_get_o`` without the base matmuls
+    (:285-299, :393-415): copy each adapter's tokens into the padded batch,
+    ``bmm(bmm(emb, A), B)``, then ``y[tokens] += delta * scaling``.
+
+    ``A[i][p]``: (H, r_i), ``B[i][p]``: (r_i, H_out_p) as numpy arrays for the
+    adapters that appear in the batch (the reference is handed exactly those).
+    """
+
+    def __init__(self, A, B, scaling, bins, threads=None):
+        import torch
+        if threads:
+            torch.set_num_threads(int(threads))
+        self.torch = torch
+        n = len(A)
+        max_r = max(a[0].shape[1] for a in A)
+        h = A[0][0].shape[0]
+        self.h_out = [B[0][p].shape[1] for p in range(4)]
+        self.pad_A = [torch.zeros((n, h, max_r), dtype=torch.float32) for _ in range(4)]
+        self.pad_B = [torch.zeros((n, max_r, self.h_out[p]), dtype=torch.float32) for p in range(4)]
+        for i in range(n):
+            r = A[i][0].shape[1]
+            for p in range(4):
+                self.pad_A[p][i, :, :r] = torch.from_numpy(np.ascontiguousarray(A[i][p]))
+                self.pad_B[p][i, :r, :] = torch.from_numpy(np.ascontiguousarray(B[i][p]))
+        bins = np.asarray(bins)
+        self.idx = [torch.from_numpy(np.nonzero(bins == i)[0]) for i in range(n)]
+        self.scaling = [float(s) for s in scaling]
+        max_tok = max(int(ix.numel()) for ix in self.idx)
+        self.emb = torch.zeros((n, max_tok, h), dtype=torch.float32)
+
+    def _proj(self, p, x, y):
+        torch = self.torch
+        for i, ix in enumerate(self.idx):
+            self.emb[i, : ix.numel()] = x[ix]
+        delta = torch.bmm(torch.bmm(self.emb, self.pad_A[p]), self.pad_B[p])
+        for i, ix in enumerate(self.idx):
+            y[ix] += delta[i, : ix.numel()] * self.scaling[i]
+
+    def decode(self, x_in, x_att, ys):
+        """q, k, v from ``x_in``; o from ``x_att``; ``ys`` are updated in place."""
+        for p in range(3):
+            self._proj(p, x_in, ys[p])
+        self._proj(3, x_att, ys[3])

@@ -1,11 +1,26 @@
 // Decode-time batched gather matrix-vector products over the paged adapter
 // pool: shrink (x[H] -> delta[r]) and expand (delta[r] -> y[H_out] +=).
 //
-// Both kernels are bandwidth kernels.  One workgroup of 8 wavefronts is
-// launched per (token, 64 KiB slice of the token's adapter weights); tokens of
-// the same adapter are merged into runs so a slice is fetched once per run.
-// Every wavefront owns 8 KiB of weights (one A row / 8 contiguous 1 KiB pieces
-// of B^T) and issues all of its 16-byte loads before it waits for any.
+// Both kernels are bandwidth kernels and, at decode sizes, latency kernels: a
+// call moves a few tens of MB, so what counts is how many DEPENDENT memory
+// round trips separate kernel start from the weight loads, and how many bytes
+// are in flight at once.  The unit of work is one pool page per wavefront task
+// (an A row for shrink, one page of the flattened B^T for expand): a wavefront
+// issues all 16-byte loads of its pages before it waits for any.  A workgroup
+// covers one "item": 8 consecutive rows/pages of the projection blocks of one
+// "run" (up to kTT tokens that share an adapter, so the pages are fetched once
+// for all of them); the run's activations are staged once in LDS.
+//   single projection: 4 wavefronts x 2 pages;   q/k/v fused: 8 wavefronts x 3 pages.
+//
+// Two ways to find the items:
+//  * stateless (dispatch_bgmv as the reference calls it): a workgroup per
+//    (token, 8-row block); every wavefront scans the per-token adapter ids
+//    itself (ballots, no barrier), then walks bins -> a_len/a_start -> a_loc ->
+//    page: four dependent round trips, and blocks beyond the adapter's rank or
+//    of tokens that do not lead a run exit;
+//  * planned: slora_bgmv_plan_build() writes the item list (tokens and page
+//    ids) once per batch; every later call launches exactly one workgroup per
+//    item, reads the item in one round trip and goes straight to the weights.
 //
 // Replaces slora/csrc/bgmv/bgmv_impl.cuh:14-241 of the reference.
 
@@ -15,10 +30,10 @@
 namespace slora {
 namespace {
 
-constexpr int kThreads = 512;
-constexpr int kWaves = kThreads / kWave;  // 8
 constexpr int kTT = 4;                    // most tokens merged into one run
-constexpr int kVecPerPass = 8;            // 16-byte vectors a lane holds per pass over a row
+constexpr int kRB = 8;                    // rows / pages per item
+constexpr int kVecPerPass = 8;            // 16-byte vectors a lane holds per pass over a page
+constexpr int kPassElems = kVecPerPass * kWave * 8;  // 4096 elements
 
 struct Tables {
   const int64_t* a_start;
@@ -36,107 +51,271 @@ __device__ __forceinline__ int64_t lookup_page(const Tables& t, int64_t li) {
 }
 
 // ---------------------------------------------------------------------------
+// plan: the items of a batch
+// ---------------------------------------------------------------------------
+// int32 words: a 16-word header, then one 48-word (192-byte) record per item:
+//   [0] adapter  [1] rank  [2] n_tok  [3] j0 = first row of the item
+//   [4..8)   token indices
+//   [8..40)  page id of a_loc entry p*rank + j0 + i at [8 + p*8 + i]  (p = q,k,v,o; -1 = none)
+//   [40..42) a_start[adapter] (int64)
+//   [42]     1 if this is the run's last stored item and rank > rank_cap (rows the plan does not list)
+constexpr int kPlanMagic = 0x534c5032;  // "SLP2"
+constexpr int kPlanHeaderWords = 16;
+constexpr int kItemWords = 48;
+enum { PH_MAGIC = 0, PH_NITEMS = 1, PH_MAXRANK = 2, PH_BATCH = 3, PH_TT = 4, PH_RANKCAP = 5, PH_NRUNS = 6 };
+enum { IT_ADAPTER = 0, IT_RANK = 1, IT_NTOK = 2, IT_J0 = 3, IT_TOK = 4, IT_PAGES = 8, IT_BASE = 40, IT_MORE = 42 };
+
+struct Item {
+  int64_t a;     // adapter
+  int64_t base;  // a_start[a]
+  int r;         // rank
+  int n_tok;     // tokens in the run (0: nothing to do)
+  int j0;        // first row / page of the item inside each projection block
+  int more;      // rows beyond the listed ones exist (rank > rank_cap)
+  int tok[kTT];  // token indices
+};
+
+__device__ __forceinline__ int item_token(const Item& it, int t) {
+  int tk = 0;
+#pragma unroll
+  for (int k = 0; k < kTT; ++k)
+    if (k == t) tk = it.tok[k];
+  return tk;
+}
+
+// Stateless discovery by ONE wavefront: which tokens share token b's adapter,
+// is b the first of a run of kTT, and who are the others.  No LDS, no barrier;
+// every wavefront of the workgroup computes the same answer.  The adapter ids
+// are loaded 512 at a time so the loads of a group overlap.
+__device__ __forceinline__ void discover_run(const Tables& t, int batch, int b, Item& it) {
+  const int lane = threadIdx.x & 63;
+  it.n_tok = 0;
+  it.r = 0;
+  it.more = 0;
+  constexpr int kGroup = 8;  // chunks of 64 ids loaded together
+  const int64_t a = t.bins[b];
+  int64_t v[kGroup];
+#pragma unroll
+  for (int c = 0; c < kGroup; ++c) {
+    const int tkn = c * kWave + lane;
+    v[c] = tkn < batch ? t.bins[tkn] : (int64_t)-1;
+  }
+  if ((uint64_t)a >= (uint64_t)t.n_adapters) return;
+  // in flight while the ids are compared
+  const int64_t len = t.a_len[a];
+  const int64_t base_a = t.a_start[a];
+  int pos_b = 0, n_tok = 0;
+  bool started = false;
+  for (int g0 = 0; g0 < batch; g0 += kGroup * kWave) {
+    if (g0 != 0) {
+#pragma unroll
+      for (int c = 0; c < kGroup; ++c) {
+        const int tkn = g0 + c * kWave + lane;
+        v[c] = tkn < batch ? t.bins[tkn] : (int64_t)-1;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kGroup; ++c) {
+      const int base = g0 + c * kWave;
+      if (base < batch && n_tok < kTT) {
+        const int tkn = base + lane;
+        uint64_t mask = __ballot(tkn < batch && v[c] == a);
+        bool collect = started;
+        if (!started) {
+          if (base + kWave <= b) {
+            pos_b += __popcll(mask);
+          } else {
+            const int l_b = b - base;
+            pos_b += __popcll(mask & ((1ull << l_b) - 1ull));
+            if (pos_b % kTT != 0) return;  // b is not the first token of a run
+            mask &= ~((1ull << l_b) - 1ull);
+            started = true;
+            collect = true;
+          }
+        }
+        if (collect) {
+          while (mask != 0 && n_tok < kTT) {
+            const int i = __builtin_ctzll(mask);
+            mask &= mask - 1;
+#pragma unroll
+            for (int k = 0; k < kTT; ++k)
+              if (k == n_tok) it.tok[k] = base + i;
+            ++n_tok;
+          }
+        }
+      }
+    }
+    if (n_tok == kTT) break;
+  }
+  it.n_tok = n_tok;
+  it.a = a;
+  it.base = base_a;
+  it.r = len > 0 ? (int)(len >> 2) : 0;
+}
+
+// Item record of a plan.  The record's address comes from the workgroup id
+// only, so the header check and the record are one round trip.
+__device__ __forceinline__ const int* load_item(const int* __restrict__ plan, int idx, Item& it) {
+  const int* rec = plan + kPlanHeaderWords + (int64_t)idx * kItemWords;
+  const bool ok = plan[PH_MAGIC] == kPlanMagic && idx < plan[PH_NITEMS];
+  it.a = rec[IT_ADAPTER];
+  it.r = rec[IT_RANK];
+  it.n_tok = ok ? rec[IT_NTOK] : 0;
+  it.j0 = rec[IT_J0];
+  it.more = rec[IT_MORE];
+  it.base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
+#pragma unroll
+  for (int k = 0; k < kTT; ++k) it.tok[k] = rec[IT_TOK + k];
+  return rec;
+}
+
+// ---------------------------------------------------------------------------
 // shrink
 // ---------------------------------------------------------------------------
 struct ShrinkArgs {
   void* y[3];
   const void* x;
   const void* w;
+  const int* plan;  // nullptr: stateless
   Tables t;
   int64_t page_elems;
-  int batch, h_in, y_cols, nproj, qkvo0, rb_per_proj, tt;
+  int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
 };
 
-template <typename T, int TT>
-__global__ __launch_bounds__(kThreads) void bgmv_shrink_kernel(const ShrinkArgs p) {
-  extern __shared__ u32x4 s_x[];  // [run tokens][h_in / 8]
-  __shared__ uint64_t s_masks[kWaves];
-  __shared__ int s_members[TT];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// NPROJ = 1: 4 wavefronts, wavefront w takes rows j0+w and j0+w+4 of projection qkvo0.
+// NPROJ = 3: 8 wavefronts, wavefront w takes row j0+w of q, k and v.
+template <typename T, int NPROJ, bool PLANNED>
+__global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(const ShrinkArgs p) {
+  constexpr int NW = NPROJ == 3 ? 8 : 4;
+  constexpr int NTASK = NPROJ == 3 ? 3 : 2;
+  constexpr int NT = NW * kWave;
+  constexpr int kSlab = 512 / NT;  // 16-byte vectors per thread, token and 4096-element slab
+  extern __shared__ u32x4 s_x[];   // [lds_tt][h_in / 8]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  int b, rb;
-  map_block(blockIdx.x, (uint32_t)(p.rb_per_proj * p.nproj), b, rb);
-  if (b >= p.batch) return;
-  const int proj = rb / p.rb_per_proj;
-  const int j0 = (rb - proj * p.rb_per_proj) * kWaves;
-  const int64_t a = p.t.bins[b];
-  if ((uint64_t)a >= (uint64_t)p.t.n_adapters) return;
-  const int64_t len = p.t.a_len[a];
-  const int r = (int)(len >> 2);
-  const int r_eff = r < p.y_cols ? r : p.y_cols;
-  if (j0 >= r_eff) return;
-  const int n_tok = find_run<kThreads>(p.t.bins, p.batch, b, a, p.tt, s_masks, s_members);
-  if (n_tok == 0) return;
+  Item it;
+  const int* rec = nullptr;
+  if (PLANNED) {
+    rec = load_item(p.plan, blockIdx.x, it);
+  } else {
+    const int b = blockIdx.x / p.blocks;
+    discover_run(p.t, p.batch, b, it);
+    it.j0 = (blockIdx.x - b * p.blocks) * kRB;
+  }
+  if (it.n_tok <= 0) return;
+  const int r_eff = it.r < p.y_cols ? it.r : p.y_cols;
+  if (it.j0 >= r_eff) return;  // uniform over the workgroup
 
   const int nvec = p.h_in >> 3;
-  const int j = j0 + wave;
-  const u32x4* wrow = nullptr;
-  if (j < r_eff) {
-    const int64_t page = lookup_page(p.t, p.t.a_start[a] + (int64_t)r * (p.qkvo0 + proj) + j);
-    if (page >= 0) wrow = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p.w) + page * p.page_elems);
-  }
+  const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
+  int row[NTASK], proj[NTASK];
+  const u32x4* wrow[NTASK];
+  u32x4 wv[NTASK][kVecPerPass];
 
-  // first pass of this wave's row goes in flight before anything waits
-  u32x4 wv[kVecPerPass];
+  // rows jb .. jb+7 of the run: page pointers, and the first pass of this
+  // wavefront's pages goes in flight before anything waits
+  auto open_block = [&](int jb, bool from_plan) {
 #pragma unroll
-  for (int i = 0; i < kVecPerPass; ++i) {
-    const int v = i * kWave + lane;
-    wv[i] = (wrow != nullptr && v < nvec) ? wrow[v] : zero16();
-  }
-
-  __syncthreads();  // s_members
-  int members[TT];
-#pragma unroll
-  for (int t = 0; t < TT; ++t) members[t] = t < n_tok ? s_members[t] : 0;
-
-  // stage the run's activations: every row is read once per workgroup
-  const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
-  for (int t = 0; t < n_tok; ++t) {
-    const u32x4* xrow = xg + (int64_t)members[t] * nvec;
-    for (int v = tid; v < nvec; v += kThreads) s_x[t * nvec + v] = xrow[v];
-  }
-  __syncthreads();
-
-  float acc[TT];
-#pragma unroll
-  for (int t = 0; t < TT; ++t) acc[t] = 0.f;
-
-  const int vec_per_pass = kVecPerPass * kWave;
-  for (int v0 = 0; v0 < nvec; v0 += vec_per_pass) {
-    // next pass in flight while this one is consumed
-    u32x4 wn[kVecPerPass];
-    const int v1 = v0 + vec_per_pass;
-    if (v1 < nvec) {
-#pragma unroll
-      for (int i = 0; i < kVecPerPass; ++i) {
-        const int v = v1 + i * kWave + lane;
-        wn[i] = (wrow != nullptr && v < nvec) ? wrow[v] : zero16();
+    for (int i = 0; i < NTASK; ++i) {
+      const int jr = NPROJ == 3 ? wave : wave + 4 * i;  // row inside the block
+      row[i] = jb + jr;
+      proj[i] = NPROJ == 3 ? i : 0;
+      wrow[i] = nullptr;
+      if (row[i] < r_eff) {
+        int64_t page;
+        if (PLANNED && from_plan)
+          page = rec[IT_PAGES + (p.qkvo0 + proj[i]) * kRB + jr];
+        else
+          page = lookup_page(p.t, it.base + (int64_t)it.r * (p.qkvo0 + proj[i]) + row[i]);
+        if (page >= 0) wrow[i] = reinterpret_cast<const u32x4*>(wbase + page * p.page_elems);
       }
     }
-    if (wrow != nullptr) {
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        if (t < n_tok) {
+    for (int i = 0; i < NTASK; ++i)
 #pragma unroll
-          for (int i = 0; i < kVecPerPass; ++i) {
-            const int v = v0 + i * kWave + lane;
-            if (v < nvec) acc[t] = dot8<T>(wv[i], s_x[t * nvec + v], acc[t]);
+      for (int c = 0; c < kVecPerPass; ++c) {
+        const int v = c * kWave + lane;
+        wv[i][c] = (wrow[i] != nullptr && v < nvec) ? wrow[i][v] : zero16();
+      }
+  };
+  open_block(it.j0, true);
+  // a plan lists rows up to rank_cap; the run's last listed block also takes the rows beyond
+  const int j_end = (PLANNED && it.more) ? r_eff : it.j0 + kRB;
+
+  const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+  const int vec_per_pass = kVecPerPass * kWave;
+
+  for (int t0 = 0; t0 < it.n_tok; t0 += p.lds_tt) {
+    const int nt = it.n_tok - t0 < p.lds_tt ? it.n_tok - t0 : p.lds_tt;
+    if (t0 != 0) __syncthreads();
+    // stage the activations of these tokens: every row is read once per
+    // workgroup; all loads of a slab are issued before the first LDS store
+    for (int v0 = 0; v0 < nvec; v0 += kSlab * NT) {
+      u32x4 xr[kTT][kSlab];
+#pragma unroll
+      for (int t = 0; t < kTT; ++t) {
+        const u32x4* xrow = xg + (int64_t)item_token(it, t0 + t) * nvec;
+#pragma unroll
+        for (int i = 0; i < kSlab; ++i) {
+          const int v = v0 + i * NT + tid;
+          xr[t][i] = (t < nt && v < nvec) ? xrow[v] : zero16();
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < kTT; ++t)
+#pragma unroll
+        for (int i = 0; i < kSlab; ++i) {
+          const int v = v0 + i * NT + tid;
+          if (t < nt && v < nvec) s_x[t * nvec + v] = xr[t][i];
+        }
+    }
+    __syncthreads();
+
+    for (int jb = it.j0; jb < j_end; jb += kRB) {
+      if (jb != it.j0 || t0 != 0) open_block(jb, jb == it.j0);
+      float acc[NTASK][kTT];
+#pragma unroll
+      for (int i = 0; i < NTASK; ++i)
+#pragma unroll
+        for (int t = 0; t < kTT; ++t) acc[i][t] = 0.f;
+      for (int v0 = 0; v0 < nvec; v0 += vec_per_pass) {
+        if (v0 != 0) {
+#pragma unroll
+          for (int i = 0; i < NTASK; ++i)
+#pragma unroll
+            for (int c = 0; c < kVecPerPass; ++c) {
+              const int v = v0 + c * kWave + lane;
+              wv[i][c] = (wrow[i] != nullptr && v < nvec) ? wrow[i][v] : zero16();
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < kTT; ++t) {
+          if (t < nt) {
+#pragma unroll
+            for (int c = 0; c < kVecPerPass; ++c) {
+              const int v = v0 + c * kWave + lane;
+              if (v < nvec) {
+                const u32x4 xv = s_x[t * nvec + v];
+#pragma unroll
+                for (int i = 0; i < NTASK; ++i) acc[i][t] = dot8<T>(wv[i][c], xv, acc[i][t]);
+              }
+            }
           }
         }
       }
-    }
-    if (v1 < nvec) {
 #pragma unroll
-      for (int i = 0; i < kVecPerPass; ++i) wv[i] = wn[i];
-    }
-  }
-
-  uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj]);
+      for (int i = 0; i < NTASK; ++i) {
+        uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj[i]]);
 #pragma unroll
-  for (int t = 0; t < TT; ++t) {
-    if (t < n_tok) {
-      const float s = wave_sum(acc[t]);
-      if (lane == 0 && wrow != nullptr) y[(int64_t)members[t] * p.y_cols + j] = T::from_float(s);
+        for (int t = 0; t < kTT; ++t) {
+          if (t < nt) {
+            const float s = wave_sum(acc[i][t]);
+            if (lane == 0 && wrow[i] != nullptr)
+              y[(int64_t)item_token(it, t0 + t) * p.y_cols + row[i]] = T::from_float(s);
+          }
+        }
+      }
     }
   }
 }
@@ -148,162 +327,325 @@ struct ExpandArgs {
   void* y[3];
   const void* x[3];
   const void* w;
-  Tables t;
   const void* scales;
+  const int* plan;
+  Tables t;
   int64_t page_elems;
   int scales_dtype;
-  int batch, x_cols, nproj, qkvo0, tt;
+  int batch, x_cols, qkvo0, blocks, y_aligned;
   int h_out[3];
-  int blocks[3];  // workgroups per token for each projection
-  int blocks_total;
 };
 
-constexpr int kChunks = 8;  // 1 KiB pieces of B^T per wavefront
-
-// One run of tokens, adapter rank a multiple of 8.  LPO lanes share one output
-// (each holds 8 consecutive rank entries), so a wavefront-wide 16-byte load
-// covers OPW = 64 / LPO consecutive outputs = one contiguous piece of B^T.
-template <typename T, int TT, int LPO>
-__device__ __forceinline__ void expand_body(const ExpandArgs& p, int proj, int n_wg0, int r, int r_eff,
-                                            int64_t base_li, float scale, int n_tok, const int* s_members) {
+// Reduce the 8 partial sums of a pass over the LPO lanes that share an output
+// and file them, rounded to the storage type, in the wavefront's LDS strip:
+// load c covers outputs c*OPW .. c*OPW+OPW-1 of the pass, and lane c % LPO of
+// each lane group writes it.
+template <typename T, int LPO>
+__device__ __forceinline__ void file_sums(const float (&part)[kVecPerPass], float scale, int lane, uint16_t* s_strip) {
   constexpr int OPW = kWave / LPO;
-  constexpr int ROUNDS = (kChunks / LPO) > 0 ? (kChunks / LPO) : 1;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane % LPO, g = lane / LPO;
-  const int d0 = li * 8;
-  const bool d_ok = d0 < r_eff;
-  const int h_out = p.h_out[proj];
-  const int n_wave0 = n_wg0 + wave * kChunks * OPW;
-  const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
-  const uint32_t page_elems = (uint32_t)p.page_elems;
-
-  u32x4 wv[kChunks];
 #pragma unroll
-  for (int c = 0; c < kChunks; ++c) {
-    const int n = n_wave0 + c * OPW + g;
-    wv[c] = zero16();
-    if (d_ok && n < h_out) {
-      const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d0;
-      const uint32_t pg = flat / page_elems;
-      const uint32_t off = flat - pg * page_elems;
-      const int64_t page = lookup_page(p.t, base_li + pg);
-      if (page >= 0) wv[c] = ldg16(wbase + page * p.page_elems + off);
-    }
+  for (int c = 0; c < kVecPerPass; ++c) {
+    const float s = group_sum<LPO>(part[c]);
+    if (li == (c % LPO)) s_strip[c * OPW + g] = T::from_float(s * scale);
   }
+}
 
+// One page of the flattened (h_out, r) matrix B^T for one run, rank r a power
+// of two (8..128) that divides the page: r/8 lanes share an output, so a
+// wavefront-wide 16-byte load covers 512/r consecutive outputs.  The reduced,
+// scaled sums of a pass are transposed through a 1 KiB LDS strip of the
+// wavefront so that the read-modify-write of y is one 16-byte load and one
+// 16-byte store per lane and token.
+template <typename T>
+__device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const Item& it, int r_eff,
+                                            const uint16_t* wpage, int64_t flat0, float scale, uint16_t* s_strip) {
+  const int lane = threadIdx.x & 63;
+  const int r = it.r;
+  const int lg_r = __builtin_ctz((unsigned)r);
+  const int lpo = r >> 3;
+  const int d0 = (lane & (lpo - 1)) * 8;
+  const bool d_ok = d0 < r_eff;
+  const int page_elems = (int)p.page_elems;
+  const int out_per_pass = kPassElems >> lg_r;
+  const int n_page0 = (int)(flat0 >> lg_r);  // first output of this page
+  // outputs of this page: [n_page0, n_end); later pages own what lies beyond
+  const int n_page_end = n_page0 + (page_elems >> lg_r);
+  const int h_stride = p.h_out[proj];
+  const int n_end = h_stride < n_page_end ? h_stride : n_page_end;
   uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj]);
   const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x[proj]);
-  for (int t = 0; t < n_tok; ++t) {
-    const int bt = s_members[t];
-    float xs[8];
-    {
-      u32x4 xv = zero16();
-      if (d_ok) xv = ldg16(x + (int64_t)bt * p.x_cols + d0);
+
+  // first pass of the page and the run's delta fragments go in flight together
+  u32x4 wv[kVecPerPass];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // entries at or beyond r_eff do not take part (lanes are whole vectors
-        // because r_eff is a multiple of 8 on this path)
-        xs[2 * i] = T::lo(xv[i]) * scale;
-        xs[2 * i + 1] = T::hi(xv[i]) * scale;
+  for (int c = 0; c < kVecPerPass; ++c) {
+    const int e = (c * kWave + lane) * 8;
+    wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16(wpage + e) : zero16();
+  }
+  u32x4 xv[kTT];
+#pragma unroll
+  for (int t = 0; t < kTT; ++t)
+    xv[t] = (t < it.n_tok && d_ok) ? ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0) : zero16();
+
+  for (int e0 = 0; e0 < page_elems; e0 += kPassElems) {
+    if (e0 != 0) {
+#pragma unroll
+      for (int c = 0; c < kVecPerPass; ++c) {
+        const int e = e0 + (c * kWave + lane) * 8;
+        wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16(wpage + e) : zero16();
       }
     }
-    float res[ROUNDS];
+    // this lane's 8 consecutive outputs of the pass
+    const int n_mine = n_page0 + (e0 >> lg_r) + lane * 8;
+    const bool y_ok = lane * 8 < out_per_pass && n_mine < n_end;
+    u32x4 yv[kTT];
 #pragma unroll
-    for (int rd = 0; rd < ROUNDS; ++rd) res[rd] = 0.f;
+    for (int t = 0; t < kTT; ++t)
+      yv[t] = (t < it.n_tok && y_ok) ? ldg16(y + (int64_t)it.tok[t] * h_stride + n_mine) : zero16();
 #pragma unroll
-    for (int c = 0; c < kChunks; ++c) {
-      float s = dot8f<T>(wv[c], xs, 0.f);
-      s = group_sum<LPO>(s);
-      // after LPO chunks every lane of the wavefront holds exactly one output
-      if (li == (c % LPO)) res[c / LPO < ROUNDS ? c / LPO : 0] = s;
-    }
-    uint16_t* yrow = y + (int64_t)bt * h_out;
+    for (int t = 0; t < kTT; ++t) {
+      if (t < it.n_tok) {
+        float part[kVecPerPass];
 #pragma unroll
-    for (int rd = 0; rd < ROUNDS; ++rd) {
-      const int c = rd * LPO + li;
-      const int n = n_wave0 + c * OPW + g;
-      if (c < kChunks && n < h_out) yrow[n] = T::add(yrow[n], T::from_float(res[rd]));
+        for (int c = 0; c < kVecPerPass; ++c) part[c] = dot8<T>(wv[c], xv[t], 0.f);
+        switch (lpo) {
+          case 1: file_sums<T, 1>(part, scale, lane, s_strip); break;
+          case 2: file_sums<T, 2>(part, scale, lane, s_strip); break;
+          case 4: file_sums<T, 4>(part, scale, lane, s_strip); break;
+          case 8: file_sums<T, 8>(part, scale, lane, s_strip); break;
+          default: file_sums<T, 16>(part, scale, lane, s_strip); break;
+        }
+        // the same wavefront wrote the strip: its LDS operations complete in order
+        const u32x4 dv = *reinterpret_cast<const u32x4*>(s_strip + (y_ok ? lane * 8 : 0));
+        if (y_ok) {
+          u32x4 out;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint16_t lo = T::add((uint16_t)(yv[t][q] & 0xffffu), (uint16_t)(dv[q] & 0xffffu));
+            const uint16_t hi = T::add((uint16_t)(yv[t][q] >> 16), (uint16_t)(dv[q] >> 16));
+            out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+          }
+          *reinterpret_cast<u32x4*>(y + (int64_t)it.tok[t] * h_stride + n_mine) = out;
+        }
+      }
     }
   }
 }
 
-// Any rank, any alignment: one lane per output, element-wise loads.
+// Any rank, any alignment: one lane per output whose first element lies in this
+// page, element-wise loads through a_loc (an output's r elements may continue
+// on the next page).
 template <typename T>
-__device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, int n_wg0, int span, int r,
-                                              int r_eff, int64_t base_li, float scale, int n_tok,
-                                              const int* s_members) {
+__device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, const Item& it, int r_eff, int k,
+                                              int64_t base_li, float scale) {
   const int h_out = p.h_out[proj];
-  const int n_end = n_wg0 + span < h_out ? n_wg0 + span : h_out;
+  const int r = it.r;
+  const int64_t pe = p.page_elems;
+  int64_t n_lo = (k * pe + r - 1) / r, n_hi = ((k + 1) * pe + r - 1) / r;
+  if (n_hi > h_out) n_hi = h_out;
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
   uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj]);
   const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x[proj]);
-  const uint32_t page_elems = (uint32_t)p.page_elems;
-  for (int n = n_wg0 + (int)threadIdx.x; n < n_end; n += kThreads) {
-    for (int t = 0; t < n_tok; ++t) {
-      const int bt = s_members[t];
+  const int lane = threadIdx.x & 63;
+  for (int64_t n = n_lo + lane; n < n_hi; n += kWave) {
+    for (int t = 0; t < it.n_tok; ++t) {
+      const int bt = item_token(it, t);
       float acc = 0.f;
       for (int d = 0; d < r_eff; ++d) {
-        const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
-        const uint32_t pg = flat / page_elems;
-        const uint32_t off = flat - pg * page_elems;
+        const int64_t flat = n * r + d;
+        const int64_t pg = flat / pe, off = flat - pg * pe;
         const int64_t page = lookup_page(p.t, base_li + pg);
         if (page < 0) continue;
-        const float wf = T::to_float(wbase[page * p.page_elems + off]);
-        acc = __builtin_fmaf(wf, T::to_float(x[(int64_t)bt * p.x_cols + d]) * scale, acc);
+        const float wf = T::to_float(wbase[page * pe + off]);
+        acc = __builtin_fmaf(wf, T::to_float(x[(int64_t)bt * p.x_cols + d]), acc);
       }
       uint16_t* yp = y + (int64_t)bt * h_out + n;
-      *yp = T::add(*yp, T::from_float(acc));
+      *yp = T::add(*yp, T::from_float(acc * scale));
     }
   }
 }
 
-template <typename T, int TT>
-__global__ __launch_bounds__(kThreads) void bgmv_expand_kernel(const ExpandArgs p) {
-  __shared__ uint64_t s_masks[kWaves];
-  __shared__ int s_members[TT];
-
-  int b, blk;
-  map_block(blockIdx.x, (uint32_t)p.blocks_total, b, blk);
-  if (b >= p.batch) return;
-  int proj = 0;
-  if (blk >= p.blocks[0]) {
-    blk -= p.blocks[0];
-    proj = 1;
-    if (blk >= p.blocks[1]) {
-      blk -= p.blocks[1];
-      proj = 2;
-    }
-  }
-  const int64_t a = p.t.bins[b];
-  if ((uint64_t)a >= (uint64_t)p.t.n_adapters) return;
-  const int r = (int)(p.t.a_len[a] >> 2);
-  const int r_eff = r < p.x_cols ? r : p.x_cols;
-  if (r_eff <= 0) return;
-  const int nv = (r_eff + 7) >> 3;
-  int lpo = 1;
-  while (lpo < nv) lpo <<= 1;
-  const int span = kWaves * kChunks * (kWave / lpo);  // outputs per workgroup at this rank
-  const int n_wg0 = blk * span;
-  if (n_wg0 >= p.h_out[proj]) return;
-  const int n_tok = find_run<kThreads>(p.t.bins, p.batch, b, a, p.tt, s_masks, s_members);
-  if (n_tok == 0) return;
-  __syncthreads();
-
-  const int64_t base_li = p.t.a_start[a] + (int64_t)r * (p.qkvo0 + proj);
-  const float scale = load_scale(p.scales, p.scales_dtype, a);
-  const bool vec_ok = (r & 7) == 0 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0;
+// Page kk of projection `proj` for the item's run; `page` is its pool page id
+// or -2 to look it up in a_loc.
+template <typename T>
+__device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const Item& it, int r_eff, int kk,
+                                           int64_t page, float scale, bool vec_ok, uint16_t* s_strip) {
+  const int64_t base_li = it.base + (int64_t)it.r * (p.qkvo0 + proj);
   if (!vec_ok) {
-    expand_scalar<T>(p, proj, n_wg0, span, r, r_eff, base_li, scale, n_tok, s_members);
+    expand_scalar<T>(p, proj, it, r_eff, kk, base_li, scale);
     return;
   }
-  switch (lpo) {
-    case 1: expand_body<T, TT, 1>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    case 2: expand_body<T, TT, 2>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    case 4: expand_body<T, TT, 4>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    case 8: expand_body<T, TT, 8>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    case 16: expand_body<T, TT, 16>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    case 32: expand_body<T, TT, 32>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
-    default: expand_body<T, TT, 64>(p, proj, n_wg0, r, r_eff, base_li, scale, n_tok, s_members); break;
+  if (page == -2) page = lookup_page(p.t, base_li + kk);
+  if (page < 0) return;
+  const uint16_t* wpage = reinterpret_cast<const uint16_t*>(p.w) + page * p.page_elems;
+  const int64_t flat0 = (int64_t)kk * p.page_elems;
+  expand_page<T>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
+}
+
+// Expand has nothing to share between wavefronts (the delta row is 16 bytes per
+// lane), so every wavefront takes exactly one page: a workgroup is 4 wavefronts
+// = half of one projection's 8-page block of an item, and an item gets
+// 2 * NPROJ workgroups.
+template <typename T, int NPROJ, bool PLANNED>
+__global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p) {
+  constexpr int kWgPerItem = 2 * NPROJ;
+  __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint16_t* s_strip = s_out[wave];
+  const int unit = blockIdx.x / kWgPerItem;
+  const int sub = blockIdx.x - unit * kWgPerItem;
+  const int proj = sub >> 1;
+  const int jr = (sub & 1) * 4 + wave;  // page inside the item's block
+
+  Item it;
+  const int* rec = nullptr;
+  if (PLANNED) {
+    rec = load_item(p.plan, unit, it);
+  } else {
+    const int b = unit / p.blocks;
+    discover_run(p.t, p.batch, b, it);
+    it.j0 = (unit - b * p.blocks) * kRB;
+  }
+  if (it.n_tok <= 0) return;
+  const int r = it.r;
+  const int r_eff = r < p.x_cols ? r : p.x_cols;
+  if (r_eff <= 0) return;
+  const int k = it.j0 + jr;
+  // pages that hold this projection's h_out * r elements
+  int64_t n_pg = ((int64_t)p.h_out[proj] * r + p.page_elems - 1) / p.page_elems;
+  if (n_pg > r) n_pg = r;
+  // Pages the launch does not enumerate: the stateless grid stops at the delta
+  // width and a plan at rank_cap; an adapter of larger rank has more, which
+  // the wavefronts of the last enumerated block take in further rounds.
+  bool extra = false;
+  if (PLANNED)
+    extra = it.more != 0;
+  else
+    extra = it.j0 + kRB >= p.blocks * kRB;
+  if (k >= n_pg && !extra) return;
+  const float scale = load_scale(p.scales, p.scales_dtype, it.a);
+  const bool pow2 = (r & (r - 1)) == 0;
+  // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
+  const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
+                      (p.page_elems % (8 * r)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
+  if (k < n_pg) {
+    const int64_t page = PLANNED ? (int64_t)rec[IT_PAGES + (p.qkvo0 + proj) * kRB + jr] : (int64_t)-2;
+    expand_one<T>(p, proj, it, r_eff, k, page, scale, vec_ok, s_strip);
+  }
+  if (extra) {
+#pragma unroll 1
+    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, scale, vec_ok, s_strip);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// plan build: one workgroup
+// ---------------------------------------------------------------------------
+constexpr int kPlanThreads = 1024;
+constexpr int kPlanWaves = kPlanThreads / kWave;
+
+// exclusive prefix sum of `v` over the workgroup; *total receives the sum
+__device__ __forceinline__ int block_exclusive_scan(int v, int* s_wave, int* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  if (lane == kWave - 1) s_wave[wave] = inc;
+  __syncthreads();
+  int before = 0, tot = 0;
+  for (int wv = 0; wv < kPlanWaves; ++wv) {
+    const int c = s_wave[wv];
+    if (wv < wave) before += c;
+    tot += c;
+  }
+  __syncthreads();
+  *total = tot;
+  return before + inc - v;
+}
+
+__global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict__ plan, Tables t, int batch,
+                                                                 int rank_cap, int max_items) {
+  __shared__ int s_wave[kPlanWaves];
+  __shared__ int s_max_rank;
+  const int tid = threadIdx.x;
+  if (tid == 0) s_max_rank = 0;
+  __syncthreads();
+  int item_base = 0, run_base = 0;
+  for (int b0 = 0; b0 < batch; b0 += kPlanThreads) {
+    const int b = b0 + tid;
+    bool leader = false;
+    int64_t a = -1;
+    int r = 0;
+    if (b < batch) {
+      a = t.bins[b];
+      if ((uint64_t)a < (uint64_t)t.n_adapters) {
+        int pos = 0;
+        for (int q = 0; q < b; ++q) pos += (t.bins[q] == a) ? 1 : 0;
+        const int64_t len = t.a_len[a];
+        r = len > 0 ? (int)(len >> 2) : 0;
+        leader = (pos % kTT) == 0 && r > 0;
+      }
+    }
+    const int r_listed = r < rank_cap ? r : rank_cap;
+    const int n_it = leader ? (r_listed + kRB - 1) / kRB : 0;
+    int tot_items = 0, tot_runs = 0;
+    const int first = item_base + block_exclusive_scan(n_it, s_wave, &tot_items);
+    (void)block_exclusive_scan(leader ? 1 : 0, s_wave, &tot_runs);
+    if (leader) {
+      const int64_t base = t.a_start[a];
+      int toks[kTT];
+      int n = 0;
+      for (int q = b; q < batch && n < kTT; ++q)
+        if (t.bins[q] == a) toks[n++] = q;
+      for (int q = n; q < kTT; ++q) toks[q] = 0;
+      for (int i = 0; i < n_it; ++i) {
+        if (first + i >= max_items) break;
+        int* rec = plan + kPlanHeaderWords + (int64_t)(first + i) * kItemWords;
+        rec[IT_ADAPTER] = (int)a;
+        rec[IT_RANK] = r;
+        rec[IT_NTOK] = n;
+        rec[IT_J0] = i * kRB;
+        for (int q = 0; q < kTT; ++q) rec[IT_TOK + q] = toks[q];
+        rec[IT_BASE] = (int)(uint32_t)(uint64_t)base;
+        rec[IT_BASE + 1] = (int)(uint32_t)((uint64_t)base >> 32);
+        rec[IT_MORE] = (i == n_it - 1 && r > rank_cap) ? 1 : 0;
+        for (int q = IT_MORE + 1; q < kItemWords; ++q) rec[q] = 0;
+      }
+      atomicMax(&s_max_rank, r);
+    }
+    item_base += tot_items;
+    run_base += tot_runs;
+  }
+  __syncthreads();
+  const int n_items = item_base < max_items ? item_base : max_items;
+  // page ids, all threads over (item, projection, row)
+  for (int64_t i = tid; i < (int64_t)n_items * 4 * kRB; i += kPlanThreads) {
+    const int item = (int)(i / (4 * kRB));
+    const int e = (int)(i - (int64_t)item * (4 * kRB));
+    const int proj = e / kRB, jr = e - proj * kRB;
+    int* rec = plan + kPlanHeaderWords + (int64_t)item * kItemWords;
+    const int r = rec[IT_RANK];
+    const int j = rec[IT_J0] + jr;
+    int page = -1;
+    if (j < r) {
+      const int64_t base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
+      const int64_t pg = lookup_page(t, base + (int64_t)proj * r + j);
+      page = pg >= 0 && pg <= 0x7fffffffLL ? (int)pg : -1;
+    }
+    rec[IT_PAGES + e] = page;
+  }
+  if (tid == 0) {
+    plan[PH_MAGIC] = kPlanMagic;
+    plan[PH_NITEMS] = n_items;
+    plan[PH_MAXRANK] = s_max_rank;
+    plan[PH_BATCH] = batch;
+    plan[PH_TT] = kTT;
+    plan[PH_RANKCAP] = rank_cap;
+    plan[PH_NRUNS] = run_base;
   }
 }
 
@@ -327,17 +669,18 @@ int fill_tables(Tables& t, const slora_tables* in, const int64_t* bins, int64_t 
 constexpr size_t kLdsSoftLimit = 64 * 1024;
 constexpr size_t kLdsHardLimit = 160 * 1024 - 256;
 
-template <typename T>
-int launch_shrink(const ShrinkArgs& a, hipStream_t stream) {
-  ShrinkArgs p = a;
-  // as many tokens per run as fit the LDS budget
+int64_t plan_max_items(int64_t batch, int64_t rank_cap) { return batch * ((rank_cap + kRB - 1) / kRB); }
+
+template <typename T, int NPROJ, bool PLANNED>
+int launch_shrink(ShrinkArgs p, int64_t grid, hipStream_t stream) {
+  // as many tokens staged at once as fit a modest LDS budget
   const size_t row_bytes = (size_t)p.h_in * 2;
   int tt = kTT;
-  while (tt > 1 && tt * row_bytes > kLdsSoftLimit) --tt;
+  while (tt > 1 && tt * row_bytes > 32 * 1024) --tt;
   const size_t lds = tt * row_bytes;
   if (lds > kLdsHardLimit) return SLORA_ERR_UNSUPPORTED;
-  p.tt = tt;
-  auto kernel = bgmv_shrink_kernel<T, kTT>;
+  p.lds_tt = tt;
+  auto kernel = bgmv_shrink_kernel<T, NPROJ, PLANNED>;
   if (lds > kLdsSoftLimit) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
@@ -345,40 +688,46 @@ int launch_shrink(const ShrinkArgs& a, hipStream_t stream) {
       return SLORA_ERR_LAUNCH;
     }
   }
-  const int64_t groups = (p.batch + 7) / 8;
-  const int64_t grid = groups * 8 * p.rb_per_proj * p.nproj;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kThreads), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NPROJ == 3 ? 512 : 256), lds, stream, p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+template <typename T, int NPROJ, bool PLANNED>
+int launch_expand(const ExpandArgs& p, int64_t items, hipStream_t stream) {
+  const int64_t grid = items * 2 * NPROJ;
+  if (grid <= 0) return SLORA_OK;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
 template <typename T>
-int launch_expand(const ExpandArgs& a, hipStream_t stream) {
-  ExpandArgs p = a;
-  p.tt = kTT;
-  const int nv_max = (p.x_cols + 7) / 8;
-  int lpo_max = 1;
-  while (lpo_max < nv_max) lpo_max <<= 1;
-  const int span_min = kWaves * kChunks * (kWave / lpo_max);
-  p.blocks_total = 0;
-  for (int i = 0; i < 3; ++i) {
-    p.blocks[i] = i < p.nproj ? (p.h_out[i] + span_min - 1) / span_min : 0;
-    p.blocks_total += p.blocks[i];
-  }
-  const int64_t groups = (p.batch + 7) / 8;
-  const int64_t grid = groups * 8 * p.blocks_total;
-  if (grid <= 0) return SLORA_OK;
-  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((bgmv_expand_kernel<T, kTT>), dim3((uint32_t)grid), dim3(kThreads), 0, stream, p);
-  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+int dispatch_shrink(const ShrinkArgs& p, int nproj, bool planned, int64_t grid, hipStream_t s) {
+  if (nproj == 3)
+    return planned ? launch_shrink<T, 3, true>(p, grid, s) : launch_shrink<T, 3, false>(p, grid, s);
+  return planned ? launch_shrink<T, 1, true>(p, grid, s) : launch_shrink<T, 1, false>(p, grid, s);
 }
 
-int shrink_common(void* const y[3], int nproj, int qkvo0, const void* x, const void* w, const slora_tables* tables,
-                  const int64_t* bins, int64_t batch, int64_t h_in, int64_t y_cols, int64_t page_elems,
-                  int64_t n_pages, int dtype, void* stream) {
+template <typename T>
+int dispatch_expand(const ExpandArgs& p, int nproj, bool planned, int64_t grid, hipStream_t s) {
+  if (nproj == 3)
+    return planned ? launch_expand<T, 3, true>(p, grid, s) : launch_expand<T, 3, false>(p, grid, s);
+  return planned ? launch_expand<T, 1, true>(p, grid, s) : launch_expand<T, 1, false>(p, grid, s);
+}
+
+// grid of a planned launch: the items the caller read back, else the plan's capacity
+int64_t planned_grid(int64_t n_items, int64_t batch, int64_t rank_cap) {
+  const int64_t cap = plan_max_items(batch, rank_cap);
+  return (n_items > 0 && n_items < cap) ? n_items : cap;
+}
+
+int shrink_common(const void* plan, int64_t n_items, int64_t rank_cap, void* const y[3], int nproj, int qkvo0,
+                  const void* x, const void* w, const slora_tables* tables, const int64_t* bins, int64_t batch,
+                  int64_t h_in, int64_t y_cols, int64_t page_elems, int64_t n_pages, int dtype, void* stream) {
   if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
-  if (batch < 0 || h_in < 0 || y_cols < 0 || page_elems < 0) return SLORA_ERR_BAD_SHAPE;
+  if (batch < 0 || h_in < 0 || y_cols < 0 || page_elems < 0 || n_items < 0) return SLORA_ERR_BAD_SHAPE;
   if (qkvo0 < 0 || qkvo0 + nproj > 4) return SLORA_ERR_BAD_SHAPE;
   if (batch == 0 || y_cols == 0) return SLORA_OK;
   ShrinkArgs p{};
@@ -394,25 +743,28 @@ int shrink_common(void* const y[3], int nproj, int qkvo0, const void* x, const v
   for (int i = 0; i < 3; ++i) p.y[i] = i < nproj ? y[i] : nullptr;
   p.x = x;
   p.w = w;
+  p.plan = static_cast<const int*>(plan);
   p.page_elems = page_elems;
   p.batch = (int)batch;
   p.h_in = (int)h_in;
   p.y_cols = (int)y_cols;
-  p.nproj = nproj;
   p.qkvo0 = qkvo0;
-  p.rb_per_proj = (int)((y_cols + kWaves - 1) / kWaves);
+  p.blocks = (int)((y_cols + kRB - 1) / kRB);
+  const bool planned = plan != nullptr;
+  const int64_t grid = planned ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_shrink<F16>(p, s) : launch_shrink<BF16>(p, s);
+  return dtype == SLORA_DTYPE_F16 ? dispatch_shrink<F16>(p, nproj, planned, grid, s)
+                                  : dispatch_shrink<BF16>(p, nproj, planned, grid, s);
 }
 
-int expand_common(void* const y[3], const void* const x[3], const int64_t h_out[3], int nproj, int qkvo0,
-                  const void* w, const slora_tables* tables, const int64_t* bins, const void* scales,
-                  int scales_dtype, int64_t batch, int64_t x_cols, int64_t page_elems, int64_t n_pages, int dtype,
-                  void* stream) {
+int expand_common(const void* plan, int64_t n_items, int64_t rank_cap, void* const y[3], const void* const x[3],
+                  const int64_t h_out[3], int nproj, int qkvo0, const void* w, const slora_tables* tables,
+                  const int64_t* bins, const void* scales, int scales_dtype, int64_t batch, int64_t x_cols,
+                  int64_t page_elems, int64_t n_pages, int dtype, void* stream) {
   if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
   if (scales_dtype != SLORA_DTYPE_F16 && scales_dtype != SLORA_DTYPE_BF16 && scales_dtype != SLORA_DTYPE_F32)
     return SLORA_ERR_BAD_DTYPE;
-  if (batch < 0 || x_cols < 0 || page_elems < 0) return SLORA_ERR_BAD_SHAPE;
+  if (batch < 0 || x_cols < 0 || page_elems < 0 || n_items < 0) return SLORA_ERR_BAD_SHAPE;
   for (int i = 0; i < nproj; ++i)
     if (h_out[i] < 0) return SLORA_ERR_BAD_SHAPE;
   if (qkvo0 < 0 || qkvo0 + nproj > 4) return SLORA_ERR_BAD_SHAPE;
@@ -431,21 +783,33 @@ int expand_common(void* const y[3], const void* const x[3], const int64_t h_out[
   if ((x_cols & 7) == 0)
     for (int i = 0; i < nproj; ++i)
       if (!aligned16(x[i])) return SLORA_ERR_ALIGNMENT;
+  int64_t h_max = 0;
   for (int i = 0; i < 3; ++i) {
     p.y[i] = i < nproj ? y[i] : nullptr;
     p.x[i] = i < nproj ? x[i] : nullptr;
     p.h_out[i] = i < nproj ? (int)h_out[i] : 0;
+    if (i < nproj && h_out[i] > h_max) h_max = h_out[i];
   }
+  if (h_max == 0) return SLORA_OK;
+  p.y_aligned = 1;
+  for (int i = 0; i < nproj; ++i)
+    if (!aligned16(y[i])) p.y_aligned = 0;
   p.w = w;
   p.scales = scales;
   p.scales_dtype = scales_dtype;
+  p.plan = static_cast<const int*>(plan);
   p.page_elems = page_elems;
   p.batch = (int)batch;
   p.x_cols = (int)x_cols;
-  p.nproj = nproj;
   p.qkvo0 = qkvo0;
+  // stateless: the rank is only known on the device; the grid covers the pages of a rank
+  // up to the delta width (an adapter uses min(rank, ceil(h_out*rank/page_elems)) pages)
+  p.blocks = (int)((x_cols + kRB - 1) / kRB);
+  const bool planned = plan != nullptr;
+  const int64_t grid = planned ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_expand<F16>(p, s) : launch_expand<BF16>(p, s);
+  return dtype == SLORA_DTYPE_F16 ? dispatch_expand<F16>(p, nproj, planned, grid, s)
+                                  : dispatch_expand<BF16>(p, nproj, planned, grid, s);
 }
 
 }  // namespace
@@ -458,15 +822,16 @@ int slora_bgmv_shrink(void* y, const void* x, const void* w, const slora_tables*
                       int dtype, void* stream) {
   void* ys[3] = {y, nullptr, nullptr};
   if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
-  return slora::shrink_common(ys, 1, qkvo, x, w, tables, bins, batch, h_in, y_cols, page_elems, n_pages, dtype,
-                              stream);
+  return slora::shrink_common(nullptr, 0, 0, ys, 1, qkvo, x, w, tables, bins, batch, h_in, y_cols, page_elems,
+                              n_pages, dtype, stream);
 }
 
 int slora_bgmv_shrink_qkv(void* y_q, void* y_k, void* y_v, const void* x, const void* w,
                           const slora_tables* tables, const int64_t* bins, int64_t batch, int64_t h_in,
                           int64_t y_cols, int64_t page_elems, int64_t n_pages, int dtype, void* stream) {
   void* ys[3] = {y_q, y_k, y_v};
-  return slora::shrink_common(ys, 3, 0, x, w, tables, bins, batch, h_in, y_cols, page_elems, n_pages, dtype, stream);
+  return slora::shrink_common(nullptr, 0, 0, ys, 3, 0, x, w, tables, bins, batch, h_in, y_cols, page_elems, n_pages,
+                              dtype, stream);
 }
 
 int slora_bgmv_expand(void* y, const void* x, const void* w, const slora_tables* tables, const int64_t* bins,
@@ -476,8 +841,8 @@ int slora_bgmv_expand(void* y, const void* x, const void* w, const slora_tables*
   const void* xs[3] = {x, nullptr, nullptr};
   const int64_t hs[3] = {h_out, 0, 0};
   if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
-  return slora::expand_common(ys, xs, hs, 1, qkvo, w, tables, bins, scales, scales_dtype, batch, x_cols, page_elems,
-                              n_pages, dtype, stream);
+  return slora::expand_common(nullptr, 0, 0, ys, xs, hs, 1, qkvo, w, tables, bins, scales, scales_dtype, batch,
+                              x_cols, page_elems, n_pages, dtype, stream);
 }
 
 int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void* x_q, const void* x_k, const void* x_v,
@@ -487,8 +852,60 @@ int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void* x_q, cons
   void* ys[3] = {y_q, y_k, y_v};
   const void* xs[3] = {x_q, x_k, x_v};
   const int64_t hs[3] = {h_out_q, h_out_k, h_out_v};
-  return slora::expand_common(ys, xs, hs, 3, 0, w, tables, bins, scales, scales_dtype, batch, x_cols, page_elems,
-                              n_pages, dtype, stream);
+  return slora::expand_common(nullptr, 0, 0, ys, xs, hs, 3, 0, w, tables, bins, scales, scales_dtype, batch, x_cols,
+                              page_elems, n_pages, dtype, stream);
+}
+
+int64_t slora_bgmv_plan_bytes(int64_t batch, int64_t rank_cap) {
+  if (batch < 0 || rank_cap <= 0 || rank_cap > SLORA_MAX_RANK || batch > (1 << 24)) return SLORA_ERR_BAD_SHAPE;
+  return 4 * ((int64_t)slora::kPlanHeaderWords + slora::plan_max_items(batch, rank_cap) * slora::kItemWords);
+}
+
+int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables, const int64_t* bins,
+                          int64_t batch, int64_t rank_cap, int64_t n_pages, void* stream) {
+  using namespace slora;
+  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
+  const int64_t need = slora_bgmv_plan_bytes(batch, rank_cap);
+  if (need < 0) return (int)need;
+  if (plan_bytes < need) return SLORA_ERR_BAD_SHAPE;
+  if (!aligned16(plan)) return SLORA_ERR_ALIGNMENT;
+  Tables t{};
+  int rc = fill_tables(t, tables, bins, n_pages);
+  if (rc != SLORA_OK) return rc;
+  const int64_t max_items = plan_max_items(batch, rank_cap);
+  if (max_items > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(bgmv_plan_kernel, dim3(1), dim3(kPlanThreads), 0, reinterpret_cast<hipStream_t>(stream),
+                     static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_bgmv_shrink_planned(const void* plan, int64_t rank_cap, int64_t n_items, int nproj, void* y0, void* y1,
+                              void* y2, const void* x, const void* w, const slora_tables* tables,
+                              const int64_t* bins, int64_t batch, int64_t h_in, int64_t y_cols, int64_t page_elems,
+                              int64_t n_pages, int qkvo, int dtype, void* stream) {
+  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (rank_cap <= 0 || rank_cap > SLORA_MAX_RANK) return SLORA_ERR_BAD_SHAPE;
+  if (nproj != 1 && nproj != 3) return SLORA_ERR_BAD_SHAPE;
+  if (nproj == 3 && qkvo != 0) return SLORA_ERR_BAD_SHAPE;
+  void* ys[3] = {y0, y1, y2};
+  return slora::shrink_common(plan, n_items, rank_cap, ys, nproj, qkvo, x, w, tables, bins, batch, h_in, y_cols,
+                              page_elems, n_pages, dtype, stream);
+}
+
+int slora_bgmv_expand_planned(const void* plan, int64_t rank_cap, int64_t n_items, int nproj, void* y0, void* y1,
+                              void* y2, const void* x0, const void* x1, const void* x2, const void* w,
+                              const slora_tables* tables, const int64_t* bins, const void* scales, int scales_dtype,
+                              int64_t batch, int64_t x_cols, int64_t h_out0, int64_t h_out1, int64_t h_out2,
+                              int64_t page_elems, int64_t n_pages, int qkvo, int dtype, void* stream) {
+  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (rank_cap <= 0 || rank_cap > SLORA_MAX_RANK) return SLORA_ERR_BAD_SHAPE;
+  if (nproj != 1 && nproj != 3) return SLORA_ERR_BAD_SHAPE;
+  if (nproj == 3 && qkvo != 0) return SLORA_ERR_BAD_SHAPE;
+  void* ys[3] = {y0, y1, y2};
+  const void* xs[3] = {x0, x1, x2};
+  const int64_t hs[3] = {h_out0, h_out1, h_out2};
+  return slora::expand_common(plan, n_items, rank_cap, ys, xs, hs, nproj, qkvo, w, tables, bins, scales,
+                              scales_dtype, batch, x_cols, page_elems, n_pages, dtype, stream);
 }
 
 }  // extern "C"

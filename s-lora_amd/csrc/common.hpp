@@ -12,6 +12,7 @@ namespace slora {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
 
@@ -25,6 +26,10 @@ struct F16 {
   static __device__ __forceinline__ uint16_t from_float(float f) {
     return __builtin_bit_cast(uint16_t, (_Float16)f);
   }
+  // c + a.lo*b.lo + a.hi*b.hi in float, straight from the packed words (v_dot2_f32_f16)
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+  }
   // y + d with both operands of the storage type, one rounding
   static __device__ __forceinline__ uint16_t add(uint16_t y, uint16_t d) {
     _Float16 s = __builtin_bit_cast(_Float16, y) + __builtin_bit_cast(_Float16, d);
@@ -36,6 +41,10 @@ struct BF16 {
   static __device__ __forceinline__ float lo(uint32_t v) { return __uint_as_float(v << 16); }
   static __device__ __forceinline__ float hi(uint32_t v) { return __uint_as_float(v & 0xffff0000u); }
   static __device__ __forceinline__ float to_float(uint16_t v) { return __uint_as_float((uint32_t)v << 16); }
+  // v_dot2_f32_bf16
+  static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+  }
   static __device__ __forceinline__ uint16_t from_float(float f) {
     uint32_t u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
@@ -64,10 +73,7 @@ __device__ __forceinline__ u32x4 zero16() { return u32x4{0u, 0u, 0u, 0u}; }
 template <typename T>
 __device__ __forceinline__ float dot8(u32x4 w, u32x4 x, float acc) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    acc = __builtin_fmaf(T::lo(w[i]), T::lo(x[i]), acc);
-    acc = __builtin_fmaf(T::hi(w[i]), T::hi(x[i]), acc);
-  }
+  for (int i = 0; i < 4; ++i) acc = T::dot2(w[i], x[i], acc);
   return acc;
 }
 

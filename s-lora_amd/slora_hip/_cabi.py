@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libslora_hip.so")
+# SLORA_HIP_LIB names another build of the same library (e.g. one compiled with other tuning constants)
+_LIB_PATH = os.environ.get("SLORA_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libslora_hip.so")
 
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 
@@ -35,6 +36,12 @@ SIGNATURES = {
     "slora_bgmv_shrink_qkv": (_I, [_P, _P, _P, _P, _P, _TP, _P, _I64, _I64, _I64, _I64, _I64, _I, _P]),
     "slora_bgmv_expand_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64, _I64, _I64, _I64, _I64,
                                    _I64, _I64, _I, _P]),
+    "slora_bgmv_plan_bytes": (_I64, [_I64, _I64]),
+    "slora_bgmv_plan_build": (_I, [_P, _I64, _TP, _P, _I64, _I64, _I64, _P]),
+    "slora_bgmv_shrink_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _TP, _P, _I64, _I64, _I64, _I64, _I64,
+                                       _I, _I, _P]),
+    "slora_bgmv_expand_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64, _I64,
+                                       _I64, _I64, _I64, _I64, _I64, _I, _I, _P]),
     "slora_sgmm_shrink": (_I, [_P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I, _I, _P]),
     "slora_sgmm_expand": (_I, [_P, _P, _P, _TP, _P, _I, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,

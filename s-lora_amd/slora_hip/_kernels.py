@@ -72,7 +72,49 @@ def _validate_common(w, start_indicies, lora_ranks, loc_indicies, indicies, lora
                                f"{lora_scales.numel()} vs {start_indicies.numel()}")
 
 
-def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales) -> None:
+class BgmvPlan:
+    """Device-side list of the batch's runs (tokens that share an adapter) and
+    their page ids, built once per decode step and passed as ``plan=`` to the
+    ``dispatch_bgmv*`` calls of that step.  Valid while ``indicies`` and the
+    adapter tables keep their contents."""
+
+    def __init__(self, buf, rank_cap, batch, n_items=0, max_rank=0, n_runs=0):
+        self.buf = buf
+        self.rank_cap = int(rank_cap)
+        self.batch = int(batch)
+        self.n_items = int(n_items)    # 0 = not read back: launches are sized for the plan's capacity
+        self.max_rank = int(max_rank)
+        self.n_runs = int(n_runs)
+
+
+def make_plan(start_indicies, lora_ranks, loc_indicies, indicies, rank_cap, n_pages, readback=True) -> BgmvPlan:
+    """Build the plan for one batch.  ``rank_cap`` is the width of the shrink
+    outputs (``max_lora_dim`` of lora_unordered_batch_infer.py:21-22),
+    ``n_pages`` the number of pages of the pool buffers.  ``readback=True``
+    copies the item count to the host (one synchronisation per step) so later
+    launches have exactly one workgroup per item."""
+    for t, n in ((start_indicies, "start_indicies"), (lora_ranks, "lora_ranks"), (loc_indicies, "loc_indicies"),
+                 (indicies, "indicies")):
+        _check_input(t, n)
+        _check_index(t, n)
+    lib = _cabi.load_library()
+    batch = indicies.numel()
+    nbytes = lib.slora_bgmv_plan_bytes(batch, int(rank_cap))
+    if nbytes < 0:
+        _cabi.check(int(nbytes), "make_plan", f"(batch={batch} rank_cap={rank_cap})")
+    buf = torch.empty((max(int(nbytes), 64) + 3) // 4, dtype=torch.int32, device=indicies.device)
+    tables = _tables(start_indicies, lora_ranks, loc_indicies)
+    rc = lib.slora_bgmv_plan_build(buf.data_ptr(), buf.numel() * 4, C.byref(tables), indicies.data_ptr(), batch,
+                                   int(rank_cap), int(n_pages), _stream(indicies))
+    _cabi.check(rc, "make_plan")
+    plan = BgmvPlan(buf, rank_cap, batch)
+    if readback and batch > 0:
+        head = buf[:8].cpu()
+        plan.n_items, plan.max_rank, plan.n_runs = int(head[1]), int(head[2]), int(head[6])
+    return plan
+
+
+def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales, plan=None) -> None:
     """``y`` (in place) from ``x`` and the paged adapter pool ``w``.
 
     ``x.size(1) >= y.size(1)``: shrink, ``y[b, :r] = x[b] @ A`` (overwrite,
@@ -81,6 +123,9 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     ``r = lora_ranks[a] // 4``; A rows / B pages are
     ``w[loc_indicies[start_indicies[a] + r*qkvo + i]]`` (direction rule:
     slora/csrc/bgmv/bgmv_impl.cuh:221).
+
+    ``plan`` (keyword, optional, not in the reference): a ``BgmvPlan`` from
+    ``make_plan`` for this batch; same results, fewer dependent table reads.
     """
     _check_input(y, "y")
     _check_input(x, "x")
@@ -103,19 +148,35 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     page_elems = w.size(1) * w.size(2)
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
     code = _DTYPE_CODE[x.dtype]
+    if plan is not None and plan.batch != batch:
+        raise RuntimeError(f"plan was built for {plan.batch} tokens, this call has {batch}")
     if h_in < h_out:
-        rc = lib.slora_bgmv_expand(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
-                                   lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype], batch, h_in, h_out,
-                                   page_elems, w.size(0), qkvo, code, _stream(x))
+        if plan is not None:
+            rc = lib.slora_bgmv_expand_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 1, y.data_ptr(), None,
+                                               None, x.data_ptr(), None, None, w.data_ptr(), C.byref(tables),
+                                               indicies.data_ptr(), lora_scales.data_ptr(),
+                                               _DTYPE_CODE[lora_scales.dtype], batch, h_in, h_out, 0, 0, page_elems,
+                                               w.size(0), qkvo, code, _stream(x))
+        else:
+            rc = lib.slora_bgmv_expand(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables),
+                                       indicies.data_ptr(), lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype],
+                                       batch, h_in, h_out, page_elems, w.size(0), qkvo, code, _stream(x))
     else:
-        rc = lib.slora_bgmv_shrink(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
-                                   batch, h_in, h_out, page_elems, w.size(0), qkvo, code, _stream(x))
+        if plan is not None:
+            rc = lib.slora_bgmv_shrink_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 1, y.data_ptr(), None,
+                                               None, x.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
+                                               batch, h_in, h_out, page_elems, w.size(0), qkvo, code, _stream(x))
+        else:
+            rc = lib.slora_bgmv_shrink(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables),
+                                       indicies.data_ptr(), batch, h_in, h_out, page_elems, w.size(0), qkvo, code,
+                                       _stream(x))
     if rc == _cabi.ERR_UNSUPPORTED:
         raise RuntimeError(no_kernel)
     _cabi.check(rc, "dispatch_bgmv", f"(h_in={h_in} h_out={h_out} qkvo={qkvo})")
 
 
-def dispatch_bgmv_qkv_shrink(y_q, y_k, y_v, x, w, start_indicies, lora_ranks, loc_indicies, indicies) -> None:
+def dispatch_bgmv_qkv_shrink(y_q, y_k, y_v, x, w, start_indicies, lora_ranks, loc_indicies, indicies,
+                             plan=None) -> None:
     """The three shrink calls of one layer (qkvo = 0, 1, 2 on the same ``x``,
     lora_unordered_batch_infer.py:267-270, 287-290, 307-310) as one launch."""
     for t, n in ((y_q, "y_q"), (y_k, "y_k"), (y_v, "y_v"), (x, "x")):
@@ -133,16 +194,22 @@ def dispatch_bgmv_qkv_shrink(y_q, y_k, y_v, x, w, start_indicies, lora_ranks, lo
         raise RuntimeError(no_kernel)
     lib = _cabi.load_library()
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
-    rc = lib.slora_bgmv_shrink_qkv(y_q.data_ptr(), y_k.data_ptr(), y_v.data_ptr(), x.data_ptr(), w.data_ptr(),
-                                   C.byref(tables), indicies.data_ptr(), batch, h_in, y_cols,
-                                   w.size(1) * w.size(2), w.size(0), _DTYPE_CODE[x.dtype], _stream(x))
+    if plan is not None:
+        rc = lib.slora_bgmv_shrink_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 3, y_q.data_ptr(),
+                                           y_k.data_ptr(), y_v.data_ptr(), x.data_ptr(), w.data_ptr(),
+                                           C.byref(tables), indicies.data_ptr(), batch, h_in, y_cols,
+                                           w.size(1) * w.size(2), w.size(0), 0, _DTYPE_CODE[x.dtype], _stream(x))
+    else:
+        rc = lib.slora_bgmv_shrink_qkv(y_q.data_ptr(), y_k.data_ptr(), y_v.data_ptr(), x.data_ptr(), w.data_ptr(),
+                                       C.byref(tables), indicies.data_ptr(), batch, h_in, y_cols,
+                                       w.size(1) * w.size(2), w.size(0), _DTYPE_CODE[x.dtype], _stream(x))
     if rc == _cabi.ERR_UNSUPPORTED:
         raise RuntimeError(no_kernel)
     _cabi.check(rc, "dispatch_bgmv_qkv_shrink")
 
 
 def dispatch_bgmv_qkv_expand(y_q, y_k, y_v, x_q, x_k, x_v, w, start_indicies, lora_ranks, loc_indicies, indicies,
-                             lora_scales) -> None:
+                             lora_scales, plan=None) -> None:
     """The three expand calls of one layer (lora_unordered_batch_infer.py:271-273,
     291-295, 311-315) as one launch.  ``y_k``/``y_v`` may be narrower than
     ``y_q`` (grouped-query attention)."""
@@ -164,11 +231,19 @@ def dispatch_bgmv_qkv_expand(y_q, y_k, y_v, x_q, x_k, x_v, w, start_indicies, lo
         raise RuntimeError(no_kernel)
     lib = _cabi.load_library()
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
-    rc = lib.slora_bgmv_expand_qkv(y_q.data_ptr(), y_k.data_ptr(), y_v.data_ptr(), x_q.data_ptr(), x_k.data_ptr(),
-                                   x_v.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
-                                   lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype], batch, x_cols,
-                                   y_q.size(1), y_k.size(1), y_v.size(1), w.size(1) * w.size(2), w.size(0),
-                                   _DTYPE_CODE[x_q.dtype], _stream(x_q))
+    if plan is not None:
+        rc = lib.slora_bgmv_expand_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 3, y_q.data_ptr(),
+                                           y_k.data_ptr(), y_v.data_ptr(), x_q.data_ptr(), x_k.data_ptr(),
+                                           x_v.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
+                                           lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype], batch, x_cols,
+                                           y_q.size(1), y_k.size(1), y_v.size(1), w.size(1) * w.size(2), w.size(0), 0,
+                                           _DTYPE_CODE[x_q.dtype], _stream(x_q))
+    else:
+        rc = lib.slora_bgmv_expand_qkv(y_q.data_ptr(), y_k.data_ptr(), y_v.data_ptr(), x_q.data_ptr(), x_k.data_ptr(),
+                                       x_v.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
+                                       lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype], batch, x_cols,
+                                       y_q.size(1), y_k.size(1), y_v.size(1), w.size(1) * w.size(2), w.size(0),
+                                       _DTYPE_CODE[x_q.dtype], _stream(x_q))
     if rc == _cabi.ERR_UNSUPPORTED:
         raise RuntimeError(no_kernel)
     _cabi.check(rc, "dispatch_bgmv_qkv_expand")

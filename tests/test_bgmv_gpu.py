@@ -302,3 +302,59 @@ def test_denormal_weights_are_not_flushed(gpu):
     d_gpu, _ = run_chain(c, g, 0, 16, gpu)
     d_ref, _ = oracle_chain(c, 0, 16)
     np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,ranks,batch,h_out,rank_cap", [
+    (1024, [64, 8, 32, 16], 70, [1024, 256, 256, 1024], 64),
+    (4096, [64, 32, 16, 8, 8, 16], 256, None, 64),
+    (512, [16, 8, 64, 32], 1500, None, 64),
+    (256, [4, 12, 8, 24], 30, None, 24),       # element-wise expand path
+    (512, [64, 8, 128], 40, None, 32),          # ranks above rank_cap keep using a_loc
+])
+def test_planned_calls_equal_stateless_calls(gpu, dtype, hidden, ranks, batch, h_out, rank_cap):
+    """A plan changes how a call finds its pages, never what it computes: the
+    results must be bitwise those of the stateless calls (single and q/k/v-fused)."""
+    import slora_hip
+    from slora_hip import dispatch_bgmv, dispatch_bgmv_qkv_shrink, dispatch_bgmv_qkv_expand
+    bins = None
+    if batch == 1500:
+        bins = np.random.default_rng(3).choice(4, size=batch, p=[0.85, 0.05, 0.05, 0.05])
+    c = make_case(300 + hidden + batch, hidden, ranks, batch, dtype=dtype, h_out=h_out, zipf_alpha=1.0, bins=bins)
+    g = GpuCase(c, gpu)
+    R = max(ranks)
+    t = (g.a_start, g.a_len, g.a_loc, g.bins)
+    plan = slora_hip.make_plan(*t, rank_cap, c.n_pages)
+    assert 0 < plan.n_runs <= batch and plan.n_items >= plan.n_runs
+    assert plan.max_rank == max(ranks[i] for i in np.unique(c.bins))
+    for readback in (plan, slora_hip.make_plan(*t, rank_cap, c.n_pages, readback=False)):
+        d_s = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(4)]
+        d_p = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(4)]
+        for p in range(4):
+            dispatch_bgmv(d_s[p], g.x, g.key, *t, p, g.scales)
+            dispatch_bgmv(d_p[p], g.x, g.key, *t, p, g.scales, plan=readback)
+            assert torch.equal(d_s[p], d_p[p]), p
+        y0 = [torch.randn((batch, c.h_out[p]), dtype=g.tdt, device=gpu) for p in range(4)]
+        y_s = [v.clone() for v in y0]
+        y_p = [v.clone() for v in y0]
+        for p in range(4):
+            dispatch_bgmv(y_s[p], d_s[p], g.value, *t, p, g.scales)
+            dispatch_bgmv(y_p[p], d_s[p], g.value, *t, p, g.scales, plan=readback)
+            assert torch.equal(y_s[p], y_p[p]), p
+        # fused q/k/v with a plan
+        d_f = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+        dispatch_bgmv_qkv_shrink(d_f[0], d_f[1], d_f[2], g.x, g.key, *t, plan=readback)
+        y_f = [v.clone() for v in y0[:3]]
+        dispatch_bgmv_qkv_expand(y_f[0], y_f[1], y_f[2], d_f[0], d_f[1], d_f[2], g.value, *t, g.scales, plan=readback)
+        for p in range(3):
+            assert torch.equal(d_f[p], d_s[p]) and torch.equal(y_f[p], y_s[p]), p
+
+
+def test_plan_is_rejected_for_another_batch_size(gpu):
+    import slora_hip
+    c = make_case(19, 256, [8, 16], 12, dtype="f16")
+    g = GpuCase(c, gpu)
+    plan = slora_hip.make_plan(g.a_start, g.a_len, g.a_loc, g.bins, 16, c.n_pages)
+    d = torch.zeros((6, 16), dtype=torch.float16, device=gpu)
+    with pytest.raises(RuntimeError, match="plan was built for"):
+        slora_hip.dispatch_bgmv(d, g.x[:6], g.key, g.a_start, g.a_len, g.a_loc, g.bins[:6], 0, g.scales, plan=plan)
