@@ -36,14 +36,19 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--workload", choices=["s2", "s4", "s6"], default="s2")
-    ap.add_argument("--mode", choices=["dropin", "fused"], default="dropin",
-                    help="dropin: 8 dispatch_bgmv calls per layer as the reference issues them; "
-                         "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer)")
+    ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused"], default="planned-fused",
+                    help="dropin: 8 stateless dispatch_bgmv calls per layer exactly as the reference issues them; "
+                         "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer); "
+                         "planned*: the same with a per-step plan (built inside every timed step) passed as plan=")
+    ap.add_argument("--all-modes", action="store_true", help="also time the other modes and report them under 'modes'")
     ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
                     help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-reps", type=int, default=0, help="0 = as many as fit in about 15 s")
     ap.add_argument("--check", action="store_true", help="verify layer 0 against the oracle before timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain device copy of 256 MiB (read) + 256 MiB (write) so that a "
+                         "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) sees a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -65,41 +70,51 @@ class StepBuffers:
 
 
 def make_step(w, bufs, mode):
+    """Returns (step, shrink_sweep, expand_sweep, kernel-name suffix).  With a
+    planned mode the plan is rebuilt inside every step (one extra small launch,
+    as a caller would do once per decode step); its item count was read back
+    once when the plan was first made -- the synchronisation a caller pays per
+    step, like the reference's own ``.item()`` at lora_unordered_batch_infer.py:64."""
     import slora_hip
     bgmv = slora_hip.dispatch_bgmv
     t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
+    planned = mode.startswith("planned")
+    fused = mode.endswith("fused")
+    plan = slora_hip.make_plan(*t, w.max_rank, w.n_pages) if planned else None
+    kw = {"plan": plan} if planned else {}
 
     def shrink_sweep():
         for l in range(w.n_layers):
             for p in range(3):
-                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling)
-            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
+                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
+            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling, **kw)
 
     def expand_sweep():
         for l in range(w.n_layers):
             for p in range(3):
-                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling)
-            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
+                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling, **kw)
+            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling, **kw)
 
-    def step_dropin():
-        # call order of lora_unordered_batch_infer.py:254-318, 428-448
+    def step():
+        if planned:
+            slora_hip.rebuild_plan(plan, *t, w.n_pages)
         for l in range(w.n_layers):
-            for p in range(3):
-                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling)
-                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling)
-            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
-            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
+            if fused:
+                slora_hip.dispatch_bgmv_qkv_shrink(bufs.delta[0], bufs.delta[1], bufs.delta[2], bufs.x_in[l],
+                                                   w.key_buffer[l], *t, **kw)
+                slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0],
+                                                   bufs.delta[1], bufs.delta[2], w.value_buffer[l], *t, w.a_scaling,
+                                                   **kw)
+            else:
+                # call order of lora_unordered_batch_infer.py:254-318
+                for p in range(3):
+                    bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
+                    bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling, **kw)
+            # o projection, lora_unordered_batch_infer.py:428-448
+            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling, **kw)
+            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling, **kw)
 
-    def step_fused():
-        for l in range(w.n_layers):
-            slora_hip.dispatch_bgmv_qkv_shrink(bufs.delta[0], bufs.delta[1], bufs.delta[2], bufs.x_in[l],
-                                               w.key_buffer[l], *t)
-            slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
-                                               bufs.delta[2], w.value_buffer[l], *t, w.a_scaling)
-            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling)
-            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling)
-
-    return (step_fused if mode == "fused" else step_dropin), shrink_sweep, expand_sweep
+    return step, shrink_sweep, expand_sweep
 
 
 def graphed(fn, torch):
@@ -232,6 +247,12 @@ def main():
     else:
         w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024)
     bufs = StepBuffers(w, device)
+    if args.calibrate_copy:
+        src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     step, shrink_sweep, expand_sweep = make_step(w, bufs, args.mode)
     if args.check:
         check_layer0(w, bufs, torch)
@@ -240,20 +261,33 @@ def main():
     if args.launch == "graph":
         run_step, run_shrink, run_expand = graphed(step, torch), graphed(shrink_sweep, torch), graphed(expand_sweep, torch)
 
-    # ---- the timed region: exactly K steps between two synchronisations ---------------
-    for _ in range(args.warmup):
-        run_step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        run_step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms_per_step = e0.elapsed_time(e1) / args.steps
-    ms_per_step = max(ms_per_step, wall_ms) if args.launch == "direct" else ms_per_step
+    def time_steps(fn):
+        """exactly K steps between two synchronisations; ms per step"""
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        ev_ms = e0.elapsed_time(e1) / args.steps
+        return max(ev_ms, wall_ms) if args.launch == "direct" else ev_ms
+
+    ms_per_step = time_steps(run_step)
+    other_modes = {}
+    if args.all_modes:
+        for m in ("dropin", "fused", "planned", "planned-fused"):
+            if m == args.mode:
+                continue
+            st, _, _ = make_step(w, bufs, m)
+            fn = graphed(st, torch) if args.launch == "graph" else st
+            ms = time_steps(fn)
+            other_modes[m] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1),
+                              "launches_per_step": w.n_layers * (4 if m.endswith("fused") else 8)}
 
     # ---- per-kernel launch duration: sweeps of one kernel family, same stream ---------
     n_launch = w.n_layers * 4
@@ -266,6 +300,7 @@ def main():
     expand_gbs = expand_bytes / (expand_us * 1e-6) / 1e9
     dominant = ("bgmv_expand_kernel", expand_us, expand_bytes, expand_gbs) if expand_us >= shrink_us else \
                ("bgmv_shrink_kernel", shrink_us, shrink_bytes, shrink_gbs)
+    # the sweeps above launch the single-projection kernels (planned or stateless as the mode says)
 
     step_gbs = w.step_bytes() / (ms_per_step * 1e-3) / 1e9
     out = {
@@ -289,7 +324,8 @@ def main():
             "pool_pages_per_layer": w.n_pages,
             "mode": args.mode,
             "launch": args.launch,
-            "launches_per_step": w.n_layers * (8 if args.mode == "dropin" else 4),
+            "launches_per_step": w.n_layers * (4 if args.mode.endswith("fused") else 8) +
+                                 (1 if args.mode.startswith("planned") else 0),
         },
         "step_hbm": {
             "algorithmic_bytes_per_step": w.step_bytes(),
@@ -314,6 +350,8 @@ def main():
                                    "GBps": round(expand_gbs, 1), "frac": round(expand_gbs / HBM_PEAK_GBS, 4)},
         },
     }
+    if other_modes:
+        out["modes"] = other_modes
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, bufs, torch, args.cpu_reps)
     print(json.dumps(out), flush=True)

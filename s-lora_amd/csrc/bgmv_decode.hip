@@ -26,6 +26,9 @@
 
 #include "common.hpp"
 #include "cabi_util.hpp"
+#ifdef SLORA_TIMING
+#include <stdlib.h>
+#endif
 
 namespace slora {
 namespace {
@@ -179,37 +182,54 @@ struct ShrinkArgs {
   const int* plan;  // nullptr: stateless
   Tables t;
   int64_t page_elems;
-  int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
+  int batch, h_in, y_cols, qkvo0, blocks, lds_tt, units;
+#ifdef SLORA_TIMING
+  unsigned long long* dbg;  // [grid][4] clock stamps: start, item known, weights arrived, end
+#endif
 };
 
-// NPROJ = 1: 4 wavefronts, wavefront w takes rows j0+w and j0+w+4 of projection qkvo0.
-// NPROJ = 3: 8 wavefronts, wavefront w takes row j0+w of q, k and v.
-template <typename T, int NPROJ, bool PLANNED>
-__global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(const ShrinkArgs p) {
-  constexpr int NW = NPROJ == 3 ? 8 : 4;
-  constexpr int NTASK = NPROJ == 3 ? 3 : 2;
+// 4 wavefronts; wavefront w takes rows j0+w and j0+w+4 of one projection.  A
+// q/k/v call launches three workgroups per item (projection-major, so that with
+// a multiple of 8 items all three run on the item's XCD and share its
+// activations in that L2).
+template <typename T, bool PLANNED>
+__global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
+  constexpr int NW = 4;
+  constexpr int NTASK = 2;
   constexpr int NT = NW * kWave;
   constexpr int kSlab = 512 / NT;  // 16-byte vectors per thread, token and 4096-element slab
   extern __shared__ u32x4 s_x[];   // [lds_tt][h_in / 8]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+#ifdef SLORA_TIMING
+  const unsigned long long ts0 = __builtin_amdgcn_s_memrealtime();
+#endif
 
+  const int proj = blockIdx.x / p.units;
+  const int unit = blockIdx.x - proj * p.units;
   Item it;
   const int* rec = nullptr;
   if (PLANNED) {
-    rec = load_item(p.plan, blockIdx.x, it);
+    rec = load_item(p.plan, unit, it);
   } else {
-    const int b = blockIdx.x / p.blocks;
+    const int b = unit / p.blocks;
     discover_run(p.t, p.batch, b, it);
-    it.j0 = (blockIdx.x - b * p.blocks) * kRB;
+    it.j0 = (unit - b * p.blocks) * kRB;
   }
+#ifdef SLORA_TIMING
+  if (tid == 0) {
+    p.dbg[(size_t)blockIdx.x * 4 + 0] = ts0;
+    p.dbg[(size_t)blockIdx.x * 4 + 1] = it.n_tok > 0 ? __builtin_amdgcn_s_memrealtime() : 0ull;
+    p.dbg[(size_t)blockIdx.x * 4 + 3] = 0ull;
+  }
+#endif
   if (it.n_tok <= 0) return;
   const int r_eff = it.r < p.y_cols ? it.r : p.y_cols;
   if (it.j0 >= r_eff) return;  // uniform over the workgroup
 
   const int nvec = p.h_in >> 3;
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
-  int row[NTASK], proj[NTASK];
+  int row[NTASK];
   const u32x4* wrow[NTASK];
   u32x4 wv[NTASK][kVecPerPass];
 
@@ -218,16 +238,15 @@ __global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(con
   auto open_block = [&](int jb, bool from_plan) {
 #pragma unroll
     for (int i = 0; i < NTASK; ++i) {
-      const int jr = NPROJ == 3 ? wave : wave + 4 * i;  // row inside the block
+      const int jr = wave + 4 * i;  // row inside the block
       row[i] = jb + jr;
-      proj[i] = NPROJ == 3 ? i : 0;
       wrow[i] = nullptr;
       if (row[i] < r_eff) {
         int64_t page;
         if (PLANNED && from_plan)
-          page = rec[IT_PAGES + (p.qkvo0 + proj[i]) * kRB + jr];
+          page = rec[IT_PAGES + (p.qkvo0 + proj) * kRB + jr];
         else
-          page = lookup_page(p.t, it.base + (int64_t)it.r * (p.qkvo0 + proj[i]) + row[i]);
+          page = lookup_page(p.t, it.base + (int64_t)it.r * (p.qkvo0 + proj) + row[i]);
         if (page >= 0) wrow[i] = reinterpret_cast<const u32x4*>(wbase + page * p.page_elems);
       }
     }
@@ -274,6 +293,9 @@ __global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(con
 
     for (int jb = it.j0; jb < j_end; jb += kRB) {
       if (jb != it.j0 || t0 != 0) open_block(jb, jb == it.j0);
+#ifdef SLORA_TIMING
+      if (tid == 0 && wv[0][0][0] != 0x12345678u) p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
+#endif
       float acc[NTASK][kTT];
 #pragma unroll
       for (int i = 0; i < NTASK; ++i)
@@ -304,9 +326,9 @@ __global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(con
           }
         }
       }
+      uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj]);
 #pragma unroll
       for (int i = 0; i < NTASK; ++i) {
-        uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj[i]]);
 #pragma unroll
         for (int t = 0; t < kTT; ++t) {
           if (t < nt) {
@@ -318,6 +340,9 @@ __global__ __launch_bounds__(NPROJ == 3 ? 512 : 256) void bgmv_shrink_kernel(con
       }
     }
   }
+#ifdef SLORA_TIMING
+  if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -332,7 +357,7 @@ struct ExpandArgs {
   Tables t;
   int64_t page_elems;
   int scales_dtype;
-  int batch, x_cols, qkvo0, blocks, y_aligned;
+  int batch, x_cols, qkvo0, blocks, y_aligned, units;
   int h_out[3];
 };
 
@@ -489,12 +514,12 @@ __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const 
 // 2 * NPROJ workgroups.
 template <typename T, int NPROJ, bool PLANNED>
 __global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p) {
-  constexpr int kWgPerItem = 2 * NPROJ;
   __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint16_t* s_strip = s_out[wave];
-  const int unit = blockIdx.x / kWgPerItem;
-  const int sub = blockIdx.x - unit * kWgPerItem;
+  // sub-block major: with a multiple of 8 units, every workgroup of a unit lands on XCD unit % 8
+  const int sub = blockIdx.x / p.units;
+  const int unit = blockIdx.x - sub * p.units;
   const int proj = sub >> 1;
   const int jr = (sub & 1) * 4 + wave;  // page inside the item's block
 
@@ -567,62 +592,147 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int* s_wave, int* tot
   return before + inc - v;
 }
 
+constexpr int kMaxLdsBins = 8192;  // adapter ids kept in LDS (larger batches read the rest from memory)
+constexpr int kMaxLdsRuns = 2048;  // run descriptors kept in LDS
+constexpr int kXcds = 8;
+enum { SC_ADAPTER = 0, SC_TOKEN = 1, SC_RANK = 2, SC_ITEMS = 3, SC_WORK = 4, SC_QUEUE = 5, SC_WORDS = 6 };
+
+// Builds the item list.  Runs are sorted by adapter, then cut into 8 queues of
+// equal work, one per XCD: consecutive workgroup ids go to the XCDs in turn, so
+// queue q's k-th item is stored at index k*8 + q.  All items of a run, and all
+// runs of an adapter (up to a cut), then execute on one XCD: the run's
+// activations and an adapter's pages shared by several runs are fetched by a
+// single L2.  Queues are padded to the longest with empty items.
 __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict__ plan, Tables t, int batch,
-                                                                 int rank_cap, int max_items) {
+                                                                 int rank_cap, int max_items,
+                                                                 int* __restrict__ scratch) {
+  __shared__ int s_bins[kMaxLdsBins];
+  __shared__ int s_ra[kMaxLdsRuns], s_rb[kMaxLdsRuns], s_rn[kMaxLdsRuns];
   __shared__ int s_wave[kPlanWaves];
-  __shared__ int s_max_rank;
+  __shared__ int s_max_rank, s_total;
+  __shared__ int s_qstart[kXcds], s_qlen[kXcds];
   const int tid = threadIdx.x;
-  if (tid == 0) s_max_rank = 0;
+  if (tid == 0) {
+    s_max_rank = 0;
+    s_total = 0;
+  }
+  if (tid < kXcds) {
+    s_qstart[tid] = 0x7fffffff;
+    s_qlen[tid] = 0;
+  }
+  auto adapter_of = [&](int q) -> int {
+    const int64_t a = t.bins[q];
+    return ((uint64_t)a < (uint64_t)t.n_adapters && a <= 0x7fffffffLL) ? (int)a : -1;
+  };
+  for (int i = tid; i < batch && i < kMaxLdsBins; i += kPlanThreads) s_bins[i] = adapter_of(i);
   __syncthreads();
-  int item_base = 0, run_base = 0;
+  auto bin_at = [&](int q) -> int { return q < kMaxLdsBins ? s_bins[q] : adapter_of(q); };
+
+  // ---- runs, in token order ----
+  int n_runs = 0;
   for (int b0 = 0; b0 < batch; b0 += kPlanThreads) {
     const int b = b0 + tid;
     bool leader = false;
-    int64_t a = -1;
-    int r = 0;
+    int a = -1, r = 0;
     if (b < batch) {
-      a = t.bins[b];
-      if ((uint64_t)a < (uint64_t)t.n_adapters) {
+      a = bin_at(b);
+      if (a >= 0) {
         int pos = 0;
-        for (int q = 0; q < b; ++q) pos += (t.bins[q] == a) ? 1 : 0;
+        for (int q = 0; q < b; ++q) pos += (bin_at(q) == a) ? 1 : 0;
         const int64_t len = t.a_len[a];
         r = len > 0 ? (int)(len >> 2) : 0;
         leader = (pos % kTT) == 0 && r > 0;
       }
     }
-    const int r_listed = r < rank_cap ? r : rank_cap;
-    const int n_it = leader ? (r_listed + kRB - 1) / kRB : 0;
-    int tot_items = 0, tot_runs = 0;
-    const int first = item_base + block_exclusive_scan(n_it, s_wave, &tot_items);
-    (void)block_exclusive_scan(leader ? 1 : 0, s_wave, &tot_runs);
+    int tot = 0;
+    const int idx = n_runs + block_exclusive_scan(leader ? 1 : 0, s_wave, &tot);
     if (leader) {
-      const int64_t base = t.a_start[a];
-      int toks[kTT];
-      int n = 0;
-      for (int q = b; q < batch && n < kTT; ++q)
-        if (t.bins[q] == a) toks[n++] = q;
-      for (int q = n; q < kTT; ++q) toks[q] = 0;
-      for (int i = 0; i < n_it; ++i) {
-        if (first + i >= max_items) break;
-        int* rec = plan + kPlanHeaderWords + (int64_t)(first + i) * kItemWords;
-        rec[IT_ADAPTER] = (int)a;
-        rec[IT_RANK] = r;
-        rec[IT_NTOK] = n;
-        rec[IT_J0] = i * kRB;
-        for (int q = 0; q < kTT; ++q) rec[IT_TOK + q] = toks[q];
-        rec[IT_BASE] = (int)(uint32_t)(uint64_t)base;
-        rec[IT_BASE + 1] = (int)(uint32_t)((uint64_t)base >> 32);
-        rec[IT_MORE] = (i == n_it - 1 && r > rank_cap) ? 1 : 0;
-        for (int q = IT_MORE + 1; q < kItemWords; ++q) rec[q] = 0;
+      const int r_listed = r < rank_cap ? r : rank_cap;
+      const int n_it = (r_listed + kRB - 1) / kRB;
+      int* sc = scratch + (int64_t)idx * SC_WORDS;
+      sc[SC_ADAPTER] = a;
+      sc[SC_TOKEN] = b;
+      sc[SC_RANK] = r;
+      sc[SC_ITEMS] = n_it;
+      if (idx < kMaxLdsRuns) {
+        s_ra[idx] = a;
+        s_rb[idx] = b;
+        s_rn[idx] = n_it;
       }
       atomicMax(&s_max_rank, r);
+      atomicAdd(&s_total, n_it);
     }
-    item_base += tot_items;
-    run_base += tot_runs;
+    n_runs += tot;
   }
   __syncthreads();
-  const int n_items = item_base < max_items ? item_base : max_items;
-  // page ids, all threads over (item, projection, row)
+  const int total = s_total;
+
+  // ---- order by (adapter, token): work in front of every run, then its queue ----
+  for (int rho = tid; rho < n_runs; rho += kPlanThreads) {
+    int* sc = scratch + (int64_t)rho * SC_WORDS;
+    const int a = sc[SC_ADAPTER], b = sc[SC_TOKEN], n = sc[SC_ITEMS];
+    int before = 0;
+    for (int o = 0; o < n_runs; ++o) {
+      int oa, ob, on;
+      if (o < kMaxLdsRuns) {
+        oa = s_ra[o];
+        ob = s_rb[o];
+        on = s_rn[o];
+      } else {
+        const int* so = scratch + (int64_t)o * SC_WORDS;
+        oa = so[SC_ADAPTER];
+        ob = so[SC_TOKEN];
+        on = so[SC_ITEMS];
+      }
+      if (oa < a || (oa == a && ob < b)) before += on;
+    }
+    int q = (int)(((int64_t)before * kXcds) / (total > 0 ? total : 1));
+    if (q > kXcds - 1) q = kXcds - 1;
+    sc[SC_WORK] = before;
+    sc[SC_QUEUE] = q;
+    atomicMin(&s_qstart[q], before);
+    atomicAdd(&s_qlen[q], n);
+  }
+  __syncthreads();
+  int max_len = 0;
+  for (int q = 0; q < kXcds; ++q) max_len = s_qlen[q] > max_len ? s_qlen[q] : max_len;
+  int n_items = kXcds * max_len;
+  const bool overflow = n_items > max_items;  // cannot happen with the capacity slora_bgmv_plan_bytes() reserves
+  if (overflow) n_items = 0;
+
+  // ---- records: padding first, then every run's items ----
+  for (int pos = tid; pos < n_items; pos += kPlanThreads) {
+    if (pos / kXcds >= s_qlen[pos % kXcds]) {
+      int* rec = plan + kPlanHeaderWords + (int64_t)pos * kItemWords;
+      for (int q = 0; q < kItemWords; ++q) rec[q] = q >= IT_PAGES && q < IT_BASE ? -1 : 0;
+    }
+  }
+  for (int rho = tid; rho < n_runs && !overflow; rho += kPlanThreads) {
+    const int* sc = scratch + (int64_t)rho * SC_WORDS;
+    const int a = sc[SC_ADAPTER], b = sc[SC_TOKEN], r = sc[SC_RANK], n_it = sc[SC_ITEMS];
+    const int q = sc[SC_QUEUE];
+    const int k0 = sc[SC_WORK] - s_qstart[q];
+    const int64_t base = t.a_start[a];
+    int toks[kTT];
+    int n = 0;
+    for (int c = b; c < batch && n < kTT; ++c)
+      if (bin_at(c) == a) toks[n++] = c;
+    for (int c = n; c < kTT; ++c) toks[c] = 0;
+    for (int i = 0; i < n_it; ++i) {
+      int* rec = plan + kPlanHeaderWords + ((int64_t)(k0 + i) * kXcds + q) * kItemWords;
+      rec[IT_ADAPTER] = a;
+      rec[IT_RANK] = r;
+      rec[IT_NTOK] = n;
+      rec[IT_J0] = i * kRB;
+      for (int c = 0; c < kTT; ++c) rec[IT_TOK + c] = toks[c];
+      rec[IT_BASE] = (int)(uint32_t)(uint64_t)base;
+      rec[IT_BASE + 1] = (int)(uint32_t)((uint64_t)base >> 32);
+      rec[IT_MORE] = (i == n_it - 1 && r > rank_cap) ? 1 : 0;
+      for (int c = IT_MORE + 1; c < kItemWords; ++c) rec[c] = 0;
+    }
+  }
+  __syncthreads();
+  // ---- page ids, all threads over (item, projection, row) ----
   for (int64_t i = tid; i < (int64_t)n_items * 4 * kRB; i += kPlanThreads) {
     const int item = (int)(i / (4 * kRB));
     const int e = (int)(i - (int64_t)item * (4 * kRB));
@@ -631,7 +741,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
     const int r = rec[IT_RANK];
     const int j = rec[IT_J0] + jr;
     int page = -1;
-    if (j < r) {
+    if (rec[IT_NTOK] > 0 && j < r) {
       const int64_t base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
       const int64_t pg = lookup_page(t, base + (int64_t)proj * r + j);
       page = pg >= 0 && pg <= 0x7fffffffLL ? (int)pg : -1;
@@ -645,7 +755,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
     plan[PH_BATCH] = batch;
     plan[PH_TT] = kTT;
     plan[PH_RANKCAP] = rank_cap;
-    plan[PH_NRUNS] = run_base;
+    plan[PH_NRUNS] = n_runs;
   }
 }
 
@@ -669,10 +779,16 @@ int fill_tables(Tables& t, const slora_tables* in, const int64_t* bins, int64_t 
 constexpr size_t kLdsSoftLimit = 64 * 1024;
 constexpr size_t kLdsHardLimit = 160 * 1024 - 256;
 
-int64_t plan_max_items(int64_t batch, int64_t rank_cap) { return batch * ((rank_cap + kRB - 1) / kRB); }
+// item capacity of a plan: every run's items plus the padding that evens out the 8 queues
+int64_t plan_max_items(int64_t batch, int64_t rank_cap) {
+  const int64_t per_run = (rank_cap + kRB - 1) / kRB;
+  return batch * per_run + kXcds * (per_run + 1);
+}
+// int32 words of the builder's scratch area behind the items
+int64_t plan_scratch_words(int64_t batch) { return batch * SC_WORDS; }
 
-template <typename T, int NPROJ, bool PLANNED>
-int launch_shrink(ShrinkArgs p, int64_t grid, hipStream_t stream) {
+template <typename T, bool PLANNED>
+int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
   // as many tokens staged at once as fit a modest LDS budget
   const size_t row_bytes = (size_t)p.h_in * 2;
   int tt = kTT;
@@ -680,7 +796,9 @@ int launch_shrink(ShrinkArgs p, int64_t grid, hipStream_t stream) {
   const size_t lds = tt * row_bytes;
   if (lds > kLdsHardLimit) return SLORA_ERR_UNSUPPORTED;
   p.lds_tt = tt;
-  auto kernel = bgmv_shrink_kernel<T, NPROJ, PLANNED>;
+  auto kernel = bgmv_shrink_kernel<T, PLANNED>;
+  p.units = (int)units;
+  const int64_t grid = units * nproj;
   if (lds > kLdsSoftLimit) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
@@ -690,12 +808,13 @@ int launch_shrink(ShrinkArgs p, int64_t grid, hipStream_t stream) {
   }
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(NPROJ == 3 ? 512 : 256), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(256), lds, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
 template <typename T, int NPROJ, bool PLANNED>
-int launch_expand(const ExpandArgs& p, int64_t items, hipStream_t stream) {
+int launch_expand(ExpandArgs p, int64_t items, hipStream_t stream) {
+  p.units = (int)items;
   const int64_t grid = items * 2 * NPROJ;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
@@ -704,10 +823,8 @@ int launch_expand(const ExpandArgs& p, int64_t items, hipStream_t stream) {
 }
 
 template <typename T>
-int dispatch_shrink(const ShrinkArgs& p, int nproj, bool planned, int64_t grid, hipStream_t s) {
-  if (nproj == 3)
-    return planned ? launch_shrink<T, 3, true>(p, grid, s) : launch_shrink<T, 3, false>(p, grid, s);
-  return planned ? launch_shrink<T, 1, true>(p, grid, s) : launch_shrink<T, 1, false>(p, grid, s);
+int dispatch_shrink(const ShrinkArgs& p, int nproj, bool planned, int64_t units, hipStream_t s) {
+  return planned ? launch_shrink<T, true>(p, nproj, units, s) : launch_shrink<T, false>(p, nproj, units, s);
 }
 
 template <typename T>
@@ -750,6 +867,9 @@ int shrink_common(const void* plan, int64_t n_items, int64_t rank_cap, void* con
   p.y_cols = (int)y_cols;
   p.qkvo0 = qkvo0;
   p.blocks = (int)((y_cols + kRB - 1) / kRB);
+#ifdef SLORA_TIMING
+  p.dbg = reinterpret_cast<unsigned long long*>(strtoull(getenv("SLORA_TIMING_BUF"), nullptr, 0));
+#endif
   const bool planned = plan != nullptr;
   const int64_t grid = planned ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -858,7 +978,8 @@ int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void* x_q, cons
 
 int64_t slora_bgmv_plan_bytes(int64_t batch, int64_t rank_cap) {
   if (batch < 0 || rank_cap <= 0 || rank_cap > SLORA_MAX_RANK || batch > (1 << 24)) return SLORA_ERR_BAD_SHAPE;
-  return 4 * ((int64_t)slora::kPlanHeaderWords + slora::plan_max_items(batch, rank_cap) * slora::kItemWords);
+  return 4 * ((int64_t)slora::kPlanHeaderWords + slora::plan_max_items(batch, rank_cap) * slora::kItemWords +
+              slora::plan_scratch_words(batch));
 }
 
 int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables, const int64_t* bins,
@@ -874,8 +995,9 @@ int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* ta
   if (rc != SLORA_OK) return rc;
   const int64_t max_items = plan_max_items(batch, rank_cap);
   if (max_items > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  int* scratch = static_cast<int*>(plan) + kPlanHeaderWords + max_items * kItemWords;
   hipLaunchKernelGGL(bgmv_plan_kernel, dim3(1), dim3(kPlanThreads), 0, reinterpret_cast<hipStream_t>(stream),
-                     static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items);
+                     static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items, scratch);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 

@@ -87,6 +87,19 @@ class BgmvPlan:
         self.n_runs = int(n_runs)
 
 
+def rebuild_plan(plan, start_indicies, lora_ranks, loc_indicies, indicies, n_pages) -> None:
+    """Enqueue a rebuild of ``plan`` in place for a batch of the same size (no
+    allocation, no synchronisation; the item count on the host is left as it
+    is, so use it only when the caller knows the count or left it at 0)."""
+    lib = _cabi.load_library()
+    if indicies.numel() != plan.batch:
+        raise RuntimeError(f"plan was built for {plan.batch} tokens, this batch has {indicies.numel()}")
+    tables = _tables(start_indicies, lora_ranks, loc_indicies)
+    rc = lib.slora_bgmv_plan_build(plan.buf.data_ptr(), plan.buf.numel() * 4, C.byref(tables), indicies.data_ptr(),
+                                   plan.batch, plan.rank_cap, int(n_pages), _stream(indicies))
+    _cabi.check(rc, "rebuild_plan")
+
+
 def make_plan(start_indicies, lora_ranks, loc_indicies, indicies, rank_cap, n_pages, readback=True) -> BgmvPlan:
     """Build the plan for one batch.  ``rank_cap`` is the width of the shrink
     outputs (``max_lora_dim`` of lora_unordered_batch_infer.py:21-22),
