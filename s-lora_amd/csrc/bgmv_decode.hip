@@ -732,21 +732,19 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
     }
   }
   __syncthreads();
-  // ---- page ids, all threads over (item, projection, row) ----
-  for (int64_t i = tid; i < (int64_t)n_items * 4 * kRB; i += kPlanThreads) {
-    const int item = (int)(i / (4 * kRB));
-    const int e = (int)(i - (int64_t)item * (4 * kRB));
-    const int proj = e / kRB, jr = e - proj * kRB;
+  // ---- page ids: one thread per (item, projection), its 8 lookups in flight together ----
+  for (int task = tid; task < n_items * 4; task += kPlanThreads) {
+    const int item = task >> 2, proj = task & 3;
     int* rec = plan + kPlanHeaderWords + (int64_t)item * kItemWords;
-    const int r = rec[IT_RANK];
-    const int j = rec[IT_J0] + jr;
-    int page = -1;
-    if (rec[IT_NTOK] > 0 && j < r) {
-      const int64_t base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
-      const int64_t pg = lookup_page(t, base + (int64_t)proj * r + j);
-      page = pg >= 0 && pg <= 0x7fffffffLL ? (int)pg : -1;
-    }
-    rec[IT_PAGES + e] = page;
+    const int r = rec[IT_RANK], j0 = rec[IT_J0], n_tok = rec[IT_NTOK];
+    const int64_t base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
+    int64_t pg[kRB];
+#pragma unroll
+    for (int jr = 0; jr < kRB; ++jr)
+      pg[jr] = (n_tok > 0 && j0 + jr < r) ? lookup_page(t, base + (int64_t)proj * r + j0 + jr) : (int64_t)-1;
+#pragma unroll
+    for (int jr = 0; jr < kRB; ++jr)
+      rec[IT_PAGES + proj * kRB + jr] = (pg[jr] >= 0 && pg[jr] <= 0x7fffffffLL) ? (int)pg[jr] : -1;
   }
   if (tid == 0) {
     plan[PH_MAGIC] = kPlanMagic;

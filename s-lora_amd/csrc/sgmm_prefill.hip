@@ -108,8 +108,12 @@ template <typename T>
 __global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int req = blockIdx.x / p.m_tiles;
-  const int m0 = (blockIdx.x - req * p.m_tiles) * kShrTM;
+  // consecutive workgroup ids go to the 8 XCDs in turn: keep all token tiles of a
+  // request on one XCD (request % 8) so its weight rows are fetched by one L2
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int req = (slot / p.m_tiles) * 8 + xcd;
+  const int m0 = (slot - (slot / p.m_tiles) * p.m_tiles) * kShrTM;
+  if (req >= p.t.n_requests) return;
   int64_t a;
   int r, row0, rows;
   if (!seg_lookup(p.t, req, a, r, row0, rows)) return;
@@ -159,14 +163,18 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrin
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-      for (int s = wave; s < ksteps; s += kShrWaves) {
-        const int k = s * 32 + lg * 8;
-        const bool k_ok = k < p.h_in;
-        u32x4 af[2], bf[4];
+      // This wavefront's K steps are s = wave, wave + 8, ...  A three-stage register
+      // pipeline keeps the loads of two steps in flight while a third is multiplied.
+      const int my_steps = ksteps > wave ? (ksteps - wave + kShrWaves - 1) / kShrWaves : 0;
+      auto load_step = [&](int i, u32x4 (&af)[2], u32x4 (&bf)[4]) {
+        const int k = (wave + i * kShrWaves) * 32 + lg * 8;
+        const bool k_ok = i < my_steps && k < p.h_in;
 #pragma unroll
         for (int f = 0; f < 2; ++f) af[f] = k_ok ? ldg16(xrow[f] + k) : zero16();
 #pragma unroll
         for (int t = 0; t < 4; ++t) bf[t] = (k_ok && t < n_tiles && wrow[t] != nullptr) ? ldg16(wrow[t] + k) : zero16();
+      };
+      auto mul_step = [&](const u32x4 (&af)[2], const u32x4 (&bf)[4]) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           if (t < n_tiles) {
@@ -174,6 +182,17 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrin
             for (int f = 0; f < 2; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
           }
         }
+      };
+      u32x4 a0[2], b0[4], a1[2], b1[4], a2[2], b2[4];
+      load_step(0, a0, b0);
+      load_step(1, a1, b1);
+      for (int i = 0; i < my_steps; i += 3) {
+        load_step(i + 2, a2, b2);
+        mul_step(a0, b0);
+        load_step(i + 3, a0, b0);
+        mul_step(a1, b1);
+        load_step(i + 4, a1, b1);
+        mul_step(a2, b2);
       }
       // C tile: lane holds column lr, rows 4*lg + i
       float* mine = s_part + wave * (kShrTM * kShrLd);
@@ -220,8 +239,7 @@ constexpr int kExpThreads = 256;
 constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, each 32 token rows
 constexpr int kExpTMW = 32;                     // token rows per wavefront
 constexpr int kExpTM = kExpTMW * kExpWaves;     // token rows per workgroup
-constexpr int kExpNO = 256;                     // outputs per workgroup
-constexpr int kExpOB = 64;                      // outputs per MFMA block
+constexpr int kExpOB = 64;                      // outputs per workgroup (one MFMA block)
 
 template <typename T>
 __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale, int row0,
@@ -246,10 +264,13 @@ __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t
   }
 }
 
-// KS = number of 32-wide K steps that cover the rank (1, 2 or 4)
+// One wavefront = 32 token rows x 64 outputs.  KS = number of 32-wide K steps
+// that cover the rank (1, 2 or 4).  Every load of the task (delta fragments,
+// B^T fragments, the y block) is issued before the first wait; there is no loop,
+// latency is hidden by the other wavefronts of the CU.
 template <typename T, int KS>
 __device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
-                                            int row0, int m0w, int m_cnt_w, int n0, int n_end) {
+                                            int row0, int m0w, int m_cnt_w, int nb) {
   const int lane = threadIdx.x & 63;
   const int lr = lane & 15, lg = lane >> 4;
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
@@ -257,7 +278,25 @@ __device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r
   uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
   const uint32_t page_elems = (uint32_t)p.page_elems;
 
-  // B operand: this wavefront's token rows x rank, kept for all output blocks
+  // A operand: MFMA tile t row m <-> output nb + 16*(m/4) + 4*t + (m%4), so that
+  // the four C tiles give every lane 16 consecutive outputs of one token row
+  u32x4 afrag[4][KS];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int n = nb + 16 * (lr >> 2) + 4 * t + (lr & 3);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int d = s * 32 + lg * 8;
+      afrag[t][s] = zero16();
+      if (n < p.feat_out && d < r_eff) {
+        const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
+        const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
+        const int64_t page = seg_page(p.t, base_li + pg);
+        if (page >= 0) afrag[t][s] = ldg16(wg + page * p.w_stride + off);
+      }
+    }
+  }
+  // B operand: this wavefront's token rows x rank
   u32x4 bfrag[2][KS];
   int64_t orow[2];
   bool row_ok[2];
@@ -273,70 +312,54 @@ __device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r
       bfrag[f][s] = (row_ok[f] && d < r_eff) ? ldg16(xg + row * p.x_stride + d) : zero16();
     }
   }
+  const int nl = nb + 16 * lg;  // this lane's 16 outputs start here
+  u32x4 yv[2][2];
+#pragma unroll
+  for (int f = 0; f < 2; ++f)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      yv[f][h] = (row_ok[f] && nl + 8 * h < p.feat_out) ? ldg16(og + orow[f] + nl + 8 * h) : zero16();
 
-  for (int nb = n0; nb < n_end; nb += kExpOB) {
-    // A operand: MFMA tile t row m <-> output nb + 16*(m/4) + 4*t + (m%4), so that
-    // the four C tiles give every lane 16 consecutive outputs of one token row
-    u32x4 afrag[4][KS];
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int f = 0; f < 2; ++f)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const int n = nb + 16 * (lr >> 2) + 4 * t + (lr & 3);
+      acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        const int d = s * 32 + lg * 8;
-        afrag[t][s] = zero16();
-        if (n < p.feat_out && d < r_eff) {
-          const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
-          const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
-          const int64_t page = seg_page(p.t, base_li + pg);
-          if (page >= 0) afrag[t][s] = ldg16(wg + page * p.w_stride + off);
-        }
-      }
+      for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(afrag[t][s], bfrag[f][s], acc[f][t]);
     }
-    const int nl = nb + 16 * lg;  // this lane's 16 outputs start here
-    u32x4 yv[2][2];
+  // C tile t: lane holds token column lr, output rows 4*lg + i  ->  output nl + 4*t + i
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+  for (int f = 0; f < 2; ++f) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h)
-        yv[f][h] = (row_ok[f] && nl + 8 * h < p.feat_out) ? ldg16(og + orow[f] + nl + 8 * h) : zero16();
-
-    f32x4 acc[2][4];
+    for (int h = 0; h < 2; ++h) {
+      if (row_ok[f] && nl + 8 * h < p.feat_out) {
+        u32x4 out;
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(afrag[t][s], bfrag[f][s], acc[f][t]);
-      }
-    // C tile t: lane holds token column lr, output rows 4*lg + i  ->  output nl + 4*t + i
-#pragma unroll
-    for (int f = 0; f < 2; ++f) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        if (row_ok[f] && nl + 8 * h < p.feat_out) {
-          u32x4 out;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            // elements 8h + 2q, 8h + 2q + 1 of the lane's 16 outputs
-            const int e0 = 8 * h + 2 * q;
-            const float d0 = acc[f][e0 >> 2][e0 & 3] * scale;
-            const float d1 = acc[f][(e0 + 1) >> 2][(e0 + 1) & 3] * scale;
-            const uint16_t lo = T::from_float(T::lo(yv[f][h][q]) + d0);
-            const uint16_t hi = T::from_float(T::hi(yv[f][h][q]) + d1);
-            out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
-          }
-          *reinterpret_cast<u32x4*>(og + orow[f] + nl + 8 * h) = out;
+        for (int q = 0; q < 4; ++q) {
+          // elements 8h + 2q, 8h + 2q + 1 of the lane's 16 outputs
+          const int e0 = 8 * h + 2 * q;
+          const float d0 = acc[f][e0 >> 2][e0 & 3] * scale;
+          const float d1 = acc[f][(e0 + 1) >> 2][(e0 + 1) & 3] * scale;
+          const uint16_t lo = T::from_float(T::lo(yv[f][h][q]) + d0);
+          const uint16_t hi = T::from_float(T::hi(yv[f][h][q]) + d1);
+          out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
         }
+        *reinterpret_cast<u32x4*>(og + orow[f] + nl + 8 * h) = out;
       }
     }
   }
 }
 
+// Workgroup = (request, 128-token tile, 64-output block): 4 wavefronts with 32
+// token rows each share the block's B^T fragments through the CU's L1.
 template <typename T>
 __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p) {
   const int wave = threadIdx.x >> 6;
+  // the output block is the fastest index: consecutive workgroup ids go to the 8
+  // XCDs in turn, so every XCD owns 1/8 of the output columns of ALL requests --
+  // disjoint pieces of B^T per L2 and an even share of the y traffic
   int blk = blockIdx.x;
   const int chunk = blk % p.n_chunks;
   blk /= p.n_chunks;
@@ -349,8 +372,8 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   if (r_eff <= 0) return;
   const int m_cnt = rows - m0 < kExpTM ? rows - m0 : kExpTM;
-  const int n0 = chunk * kExpNO;
-  const int n_end = n0 + kExpNO < p.feat_out ? n0 + kExpNO : p.feat_out;
+  const int n0 = chunk * kExpOB;
+  const int n_end = n0 + kExpOB < p.feat_out ? n0 + kExpOB : p.feat_out;
   const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
   const float scale = load_scale(p.scales, p.scales_dtype, a);
   if (!p.vec_ok || (r & 7) != 0 || (r_eff & 7) != 0 || r_eff > 128) {
@@ -361,11 +384,11 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   if (m0w >= rows) return;
   const int m_cnt_w = rows - m0w < kExpTMW ? rows - m0w : kExpTMW;
   if (r_eff <= 32)
-    expand_mfma<T, 1>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+    expand_mfma<T, 1>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
   else if (r_eff <= 64)
-    expand_mfma<T, 2>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+    expand_mfma<T, 2>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
   else
-    expand_mfma<T, 4>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+    expand_mfma<T, 4>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
 }
 
 // ---------------------------------------------------------------------------
@@ -405,7 +428,7 @@ int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
     }
     attr_done = true;
   }
-  const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles;
+  const int64_t grid = (int64_t)((p.t.n_requests + 7) / 8) * 8 * p.m_tiles;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, p);
@@ -490,7 +513,7 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
   p.max_rank = (int)max_rank;
   p.qkvo = qkvo;
   p.m_tiles = (int)((max_input_len + kExpTM - 1) / kExpTM);
-  p.n_chunks = (int)((feat_out + kExpNO - 1) / kExpNO);
+  p.n_chunks = (int)((feat_out + kExpOB - 1) / kExpOB);
   p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
              (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

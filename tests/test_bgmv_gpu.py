@@ -358,3 +358,34 @@ def test_plan_is_rejected_for_another_batch_size(gpu):
     d = torch.zeros((6, 16), dtype=torch.float16, device=gpu)
     with pytest.raises(RuntimeError, match="plan was built for"):
         slora_hip.dispatch_bgmv(d, g.x[:6], g.key, g.a_start, g.a_len, g.a_loc, g.bins[:6], 0, g.scales, plan=plan)
+
+
+def test_golden_fixture_decode_and_prefill(gpu):
+    """The committed closed-form fixture (tests/golden/lora_small.npz) through
+    both operator families."""
+    from test_oracle import load_golden
+    from slora_hip import dispatch_bgmv, lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand
+    g = load_golden()
+    f16 = torch.float16
+    key = torch.from_numpy(g["key"]).to(gpu)
+    value = torch.from_numpy(g["value"]).to(gpu)
+    n_pages = key.shape[0]
+    a_start, a_len, a_loc, bins = (torch.from_numpy(g[k]).to(gpu) for k in ("a_start", "a_len", "a_loc", "bins"))
+    st, ln, rq = (torch.from_numpy(g[k]).to(gpu) for k in ("b_start_loc", "b_seq_len", "b_indicies"))
+    scales = torch.from_numpy(g["scales"]).to(gpu)
+    x = torch.from_numpy(g["x"]).to(gpu)
+    T = x.shape[0]
+    for p in range(4):
+        d = torch.zeros((T, 32), dtype=f16, device=gpu)
+        dispatch_bgmv(d, x, key.view(n_pages, 4, 32), a_start, a_len, a_loc, bins, p, scales)
+        np.testing.assert_allclose(host(d), g["delta64"][p], rtol=2e-3, atol=2e-3)
+        y = torch.from_numpy(g["y0"][p]).to(gpu)
+        dispatch_bgmv(y, d, value.view(n_pages, 4, 32), a_start, a_len, a_loc, bins, p, scales)
+        np.testing.assert_allclose(host(y), g["y64"][p], rtol=1e-2, atol=1e-2)
+        o = torch.ones((T, 32), dtype=f16, device=gpu)
+        lora_get_qkvo_fwd_shrink(x, key, o, a_loc, a_start, a_len, st, ln, rq, 128, p, 32, int(g["b_seq_len"].max()))
+        np.testing.assert_allclose(host(o), g["delta64"][p], rtol=2e-3, atol=2e-3)
+        y2 = torch.from_numpy(g["y0"][p]).to(gpu)
+        lora_get_qkvo_fwd_expand(o, value, y2, scales, a_loc, a_start, a_len, st, ln, rq, 128, p, 32,
+                                 int(g["b_seq_len"].max()))
+        np.testing.assert_allclose(host(y2), g["y64"][p], rtol=1e-2, atol=1e-2)

@@ -303,3 +303,46 @@ def test_var_len_copy():
     new_start = np.array([0, 32], np.int64)
     out = O.ref_var_len_copy(old_start[keep], new_len, old_loc, new_start, int(new_len.sum()))
     assert out.tolist() == list(range(1000, 1032)) + list(range(1096, 1300))
+
+
+# ---------------------------------------------------------------------------
+# committed fixture (closed form in float64 on the dense matrices) and CPU baseline
+# ---------------------------------------------------------------------------
+def load_golden():
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lora_small.npz"))
+    return {k: g[k] for k in g.files}
+
+
+def test_oracle_matches_golden_fixture():
+    g = load_golden()
+    key, value, x = (g[k].astype(np.float32) for k in ("key", "value", "x"))
+    scales = g["scales"].astype(np.float32)
+    T = x.shape[0]
+    for p in range(4):
+        d = O.ref_bgmv_shrink(np.zeros((T, 32), np.float32), x, key, g["a_start"], g["a_len"], g["a_loc"], g["bins"], p,
+                              "f16")
+        np.testing.assert_allclose(d, g["delta64"][p], rtol=2e-3, atol=2e-3)
+        y = O.ref_bgmv_expand(g["y0"][p].astype(np.float32), d, value, g["a_start"], g["a_len"], g["a_loc"], g["bins"],
+                              p, scales, "f16")
+        np.testing.assert_allclose(y, g["y64"][p], rtol=1e-2, atol=1e-2)
+        o = O.ref_prefill_shrink(np.ones((T, 32), np.float32), x, key, g["a_loc"], g["a_start"], g["a_len"],
+                                 g["b_start_loc"], g["b_seq_len"], g["b_indicies"], p, 32, "f16")
+        np.testing.assert_allclose(o, g["delta64"][p], rtol=2e-3, atol=2e-3)
+        y2 = O.ref_prefill_expand(g["y0"][p].astype(np.float32), o, value, scales, g["a_loc"], g["a_start"], g["a_len"],
+                                  g["b_start_loc"], g["b_seq_len"], g["b_indicies"], p, 32, "f16")
+        np.testing.assert_allclose(y2, g["y64"][p], rtol=1e-2, atol=1e-2)
+
+
+def test_cpu_baseline_layer_matches_ref_bmm():
+    c = make_case(60, 128, [8, 16, 32], batch=22, dtype="f32")
+    layer = O.BmmCpuLayer(c.A, c.B, c.scales, c.bins, threads=2)
+    rng = np.random.default_rng(61)
+    x_att = rng.standard_normal((22, 128)).astype(np.float32)
+    ys = [torch.zeros((22, 128)) for _ in range(4)]
+    layer.decode(torch.from_numpy(c.x), torch.from_numpy(x_att), ys)
+    for p in range(4):
+        xin = c.x if p < 3 else x_att
+        want = O.ref_bmm(np.zeros((22, 128), np.float32), xin, [a[p] for a in c.A], [b[p] for b in c.B], c.scales,
+                         c.bins, "f32")
+        np.testing.assert_allclose(ys[p].numpy(), want, rtol=1e-4, atol=1e-5)
