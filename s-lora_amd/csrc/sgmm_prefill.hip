@@ -236,10 +236,12 @@ struct SegExpandArgs {
 };
 
 constexpr int kExpThreads = 256;
-constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, each 32 token rows
-constexpr int kExpTMW = 32;                     // token rows per wavefront
+constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, each kExpTMW token rows
+constexpr int kExpMF = 2;                       // 16-row MFMA fragments per wavefront
+constexpr int kExpTMW = 16 * kExpMF;            // token rows per wavefront
 constexpr int kExpTM = kExpTMW * kExpWaves;     // token rows per workgroup
-constexpr int kExpOB = 64;                      // outputs per workgroup (one MFMA block)
+constexpr int kExpOB = 64;                      // outputs per MFMA block
+constexpr int kExpBlocks = 1;                   // blocks a wavefront walks (512 outputs)
 
 template <typename T>
 __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale, int row0,
@@ -264,44 +266,108 @@ __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t
   }
 }
 
-// One wavefront = 32 token rows x 64 outputs.  KS = number of 32-wide K steps
-// that cover the rank (1, 2 or 4).  Every load of the task (delta fragments,
-// B^T fragments, the y block) is issued before the first wait; there is no loop,
-// latency is hidden by the other wavefronts of the CU.
+// One wavefront = kExpTMW token rows x kExpBlocks consecutive 64-output blocks.
+// KS = number of 32-wide K steps that cover the rank (1, 2 or 4).  The delta
+// fragments are loaded once per wavefront; every block then loads its B^T
+// fragments and y values together, multiplies and stores.
+//
+// MFMA orientation: rows = outputs, columns = tokens, so a lane's C values are
+// consecutive outputs of ONE token row.  The row -> output map
+//   tile t, row m  <->  output  32*(t/2) + 8*(m/4) + 4*(t%2) + (m%4)   (inside a block)
+// gives lane group g = m/4 the outputs 8g..8g+7 (tiles 0,1) and 32+8g..32+8g+7
+// (tiles 2,3): each 16-byte access of the four lane groups of a token is one
+// contiguous 64-byte run.
+template <int KS>
+struct ExpandBuf {
+  u32x4 a[4][KS];       // B^T fragments (MFMA A operand)
+  u32x4 y[kExpMF][2];   // y values this lane updates
+};
+
 template <typename T, int KS>
-__device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
-                                            int row0, int m0w, int m_cnt_w, int nb) {
+__device__ __forceinline__ void expand_load(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, int nb,
+                                            const int64_t (&orow)[kExpMF], const bool (&row_ok)[kExpMF], bool live,
+                                            ExpandBuf<KS>& buf) {
   const int lane = threadIdx.x & 63;
   const int lr = lane & 15, lg = lane >> 4;
-  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
-  uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
+  const uint16_t* og = reinterpret_cast<const uint16_t*>(p.o);
   const uint32_t page_elems = (uint32_t)p.page_elems;
-
-  // A operand: MFMA tile t row m <-> output nb + 16*(m/4) + 4*t + (m%4), so that
-  // the four C tiles give every lane 16 consecutive outputs of one token row
-  u32x4 afrag[4][KS];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
-    const int n = nb + 16 * (lr >> 2) + 4 * t + (lr & 3);
+    const int n = nb + 32 * (t >> 1) + 8 * (lr >> 2) + 4 * (t & 1) + (lr & 3);
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d = s * 32 + lg * 8;
-      afrag[t][s] = zero16();
-      if (n < p.feat_out && d < r_eff) {
+      buf.a[t][s] = zero16();
+      if (live && n < p.feat_out && d < r_eff) {
         const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
         const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
         const int64_t page = seg_page(p.t, base_li + pg);
-        if (page >= 0) afrag[t][s] = ldg16(wg + page * p.w_stride + off);
+        if (page >= 0) buf.a[t][s] = ldg16(wg + page * p.w_stride + off);
       }
     }
   }
-  // B operand: this wavefront's token rows x rank
-  u32x4 bfrag[2][KS];
-  int64_t orow[2];
-  bool row_ok[2];
 #pragma unroll
-  for (int f = 0; f < 2; ++f) {
+  for (int f = 0; f < kExpMF; ++f)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int n = nb + 32 * h + 8 * lg;
+      buf.y[f][h] = (live && row_ok[f] && n < p.feat_out) ? ldg16(og + orow[f] + n) : zero16();
+    }
+}
+
+template <typename T, int KS>
+__device__ __forceinline__ void expand_finish(const SegExpandArgs& p, float scale, int nb,
+                                              const u32x4 (&bfrag)[kExpMF][KS], const int64_t (&orow)[kExpMF],
+                                              const bool (&row_ok)[kExpMF], const ExpandBuf<KS>& buf) {
+  const int lane = threadIdx.x & 63;
+  const int lg = lane >> 4;
+  uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
+  f32x4 acc[kExpMF][4];
+#pragma unroll
+  for (int f = 0; f < kExpMF; ++f)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(buf.a[t][s], bfrag[f][s], acc[f][t]);
+    }
+  // C tile t: lane holds token column lr, rows 4*lg + i  ->  output 32*(t/2) + 8*lg + 4*(t%2) + i
+#pragma unroll
+  for (int f = 0; f < kExpMF; ++f) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int n = nb + 32 * h + 8 * lg;
+      if (row_ok[f] && n < p.feat_out) {
+        u32x4 out;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // outputs n + 2q, n + 2q + 1  <-  tile 2h + (2q)/4, element (2q)%4 and the next
+          const int e0 = 2 * q;
+          const float d0 = acc[f][2 * h + (e0 >> 2)][e0 & 3] * scale;
+          const float d1 = acc[f][2 * h + ((e0 + 1) >> 2)][(e0 + 1) & 3] * scale;
+          const uint16_t lo = T::from_float(T::lo(buf.y[f][h][q]) + d0);
+          const uint16_t hi = T::from_float(T::hi(buf.y[f][h][q]) + d1);
+          out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(og + orow[f] + n) = out;
+      }
+    }
+  }
+}
+
+template <typename T, int KS>
+__device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
+                                            int row0, int m0w, int m_cnt_w, int n0, int n_end) {
+  const int lane = threadIdx.x & 63;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
+  // MFMA B operand: this wavefront's token rows x rank, kept for all blocks
+  u32x4 bfrag[kExpMF][KS];
+  int64_t orow[kExpMF];
+  bool row_ok[kExpMF];
+#pragma unroll
+  for (int f = 0; f < kExpMF; ++f) {
     const int m = f * 16 + lr;
     row_ok[f] = m < m_cnt_w;
     const int64_t row = row0 + m0w + (row_ok[f] ? m : 0);
@@ -312,54 +378,25 @@ __device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r
       bfrag[f][s] = (row_ok[f] && d < r_eff) ? ldg16(xg + row * p.x_stride + d) : zero16();
     }
   }
-  const int nl = nb + 16 * lg;  // this lane's 16 outputs start here
-  u32x4 yv[2][2];
-#pragma unroll
-  for (int f = 0; f < 2; ++f)
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-      yv[f][h] = (row_ok[f] && nl + 8 * h < p.feat_out) ? ldg16(og + orow[f] + nl + 8 * h) : zero16();
-
-  f32x4 acc[2][4];
-#pragma unroll
-  for (int f = 0; f < 2; ++f)
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(afrag[t][s], bfrag[f][s], acc[f][t]);
-    }
-  // C tile t: lane holds token column lr, output rows 4*lg + i  ->  output nl + 4*t + i
-#pragma unroll
-  for (int f = 0; f < 2; ++f) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if (row_ok[f] && nl + 8 * h < p.feat_out) {
-        u32x4 out;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          // elements 8h + 2q, 8h + 2q + 1 of the lane's 16 outputs
-          const int e0 = 8 * h + 2 * q;
-          const float d0 = acc[f][e0 >> 2][e0 & 3] * scale;
-          const float d1 = acc[f][(e0 + 1) >> 2][(e0 + 1) & 3] * scale;
-          const uint16_t lo = T::from_float(T::lo(yv[f][h][q]) + d0);
-          const uint16_t hi = T::from_float(T::hi(yv[f][h][q]) + d1);
-          out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
-        }
-        *reinterpret_cast<u32x4*>(og + orow[f] + nl + 8 * h) = out;
-      }
-    }
+  // One buffer: the loop is not unrolled, the other wavefronts of the CU cover
+  // the two round trips (page ids, then fragments) of every block.
+#pragma unroll 1
+  for (int nb = n0; nb < n_end; nb += kExpOB) {
+    ExpandBuf<KS> buf;
+    expand_load<T, KS>(p, r, r_eff, base_li, nb, orow, row_ok, true, buf);
+    expand_finish<T, KS>(p, scale, nb, bfrag, orow, row_ok, buf);
   }
 }
 
-// Workgroup = (request, 128-token tile, 64-output block): 4 wavefronts with 32
-// token rows each share the block's B^T fragments through the CU's L1.
-template <typename T>
+// Workgroup = (request, tile of 4 * kExpTMW tokens, super-block of kExpBlocks * 64
+// outputs): its 4 wavefronts take kExpTMW token rows each and share the B^T
+// fragments through the CU's L1.
+template <typename T, int KS>
 __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p) {
   const int wave = threadIdx.x >> 6;
-  // the output block is the fastest index: consecutive workgroup ids go to the 8
-  // XCDs in turn, so every XCD owns 1/8 of the output columns of ALL requests --
-  // disjoint pieces of B^T per L2 and an even share of the y traffic
+  // the output super-block is the fastest index: consecutive workgroup ids go to
+  // the 8 XCDs in turn, so every XCD owns 1/8 of the output columns of ALL
+  // requests -- disjoint pieces of B^T per L2 and an even share of the y traffic
   int blk = blockIdx.x;
   const int chunk = blk % p.n_chunks;
   blk /= p.n_chunks;
@@ -372,8 +409,8 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   if (r_eff <= 0) return;
   const int m_cnt = rows - m0 < kExpTM ? rows - m0 : kExpTM;
-  const int n0 = chunk * kExpOB;
-  const int n_end = n0 + kExpOB < p.feat_out ? n0 + kExpOB : p.feat_out;
+  const int n0 = chunk * (kExpOB * kExpBlocks);
+  const int n_end = n0 + kExpOB * kExpBlocks < p.feat_out ? n0 + kExpOB * kExpBlocks : p.feat_out;
   const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
   const float scale = load_scale(p.scales, p.scales_dtype, a);
   if (!p.vec_ok || (r & 7) != 0 || (r_eff & 7) != 0 || r_eff > 128) {
@@ -383,12 +420,9 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   const int m0w = m0 + wave * kExpTMW;
   if (m0w >= rows) return;
   const int m_cnt_w = rows - m0w < kExpTMW ? rows - m0w : kExpTMW;
-  if (r_eff <= 32)
-    expand_mfma<T, 1>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
-  else if (r_eff <= 64)
-    expand_mfma<T, 2>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
-  else
-    expand_mfma<T, 4>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0);
+  // KS 32-wide steps cover max_rank (chosen on the host); a smaller adapter
+  // rank leaves the upper fragments zero
+  expand_mfma<T, KS>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
 }
 
 // ---------------------------------------------------------------------------
@@ -440,7 +474,12 @@ int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
   const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles * p.n_chunks;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(sgmm_expand_kernel<T>, dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
+  if (p.max_rank <= 32)
+    hipLaunchKernelGGL((sgmm_expand_kernel<T, 1>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
+  else if (p.max_rank <= 64)
+    hipLaunchKernelGGL((sgmm_expand_kernel<T, 2>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
+  else
+    hipLaunchKernelGGL((sgmm_expand_kernel<T, 4>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -513,7 +552,7 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
   p.max_rank = (int)max_rank;
   p.qkvo = qkvo;
   p.m_tiles = (int)((max_input_len + kExpTM - 1) / kExpTM);
-  p.n_chunks = (int)((feat_out + kExpOB - 1) / kExpOB);
+  p.n_chunks = (int)((feat_out + kExpOB * kExpBlocks - 1) / (kExpOB * kExpBlocks));
   p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
              (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
