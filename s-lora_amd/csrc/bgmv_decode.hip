@@ -157,19 +157,44 @@ __device__ __forceinline__ void discover_run(const Tables& t, int batch, int b, 
 }
 
 // Item record of a plan.  The record's address comes from the workgroup id
-// only, so the header check and the record are one round trip.
-__device__ __forceinline__ const int* load_item(const int* __restrict__ plan, int idx, Item& it) {
+// only.  Every field (and the page ids of rows jr0 and jr1 of projection pp) is
+// read up front and pinned in scalar registers before the first branch, so the
+// compiler cannot sink the loads below the early exits: header check, record
+// and page ids are ONE round trip of independent scalar loads.
+__device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx, int pp, int jr0, int jr1, Item& it,
+                                          int& page0, int& page1) {
   const int* rec = plan + kPlanHeaderWords + (int64_t)idx * kItemWords;
-  const bool ok = plan[PH_MAGIC] == kPlanMagic && idx < plan[PH_NITEMS];
-  it.a = rec[IT_ADAPTER];
-  it.r = rec[IT_RANK];
-  it.n_tok = ok ? rec[IT_NTOK] : 0;
-  it.j0 = rec[IT_J0];
-  it.more = rec[IT_MORE];
-  it.base = (int64_t)(((uint64_t)(uint32_t)rec[IT_BASE + 1] << 32) | (uint32_t)rec[IT_BASE]);
-#pragma unroll
-  for (int k = 0; k < kTT; ++k) it.tok[k] = rec[IT_TOK + k];
-  return rec;
+  int magic = plan[PH_MAGIC], n_items = plan[PH_NITEMS];
+  int a = rec[IT_ADAPTER], r = rec[IT_RANK], n_tok = rec[IT_NTOK], j0 = rec[IT_J0];
+  int t0 = rec[IT_TOK + 0], t1 = rec[IT_TOK + 1], t2 = rec[IT_TOK + 2], t3 = rec[IT_TOK + 3];
+  int more = rec[IT_MORE];
+  int base_lo = rec[IT_BASE], base_hi = rec[IT_BASE + 1];
+  int pg0 = rec[IT_PAGES + pp * kRB + jr0], pg1 = rec[IT_PAGES + pp * kRB + jr1];
+  asm volatile(""
+               : "+s"(magic), "+s"(n_items), "+s"(a), "+s"(r), "+s"(n_tok), "+s"(j0), "+s"(t0), "+s"(t1), "+s"(t2),
+                 "+s"(t3), "+s"(more), "+s"(base_lo), "+s"(base_hi), "+s"(pg0), "+s"(pg1));
+  static_assert(kTT == 4, "the record holds four token ids");
+  it.tok[0] = t0;
+  it.tok[1] = t1;
+  it.tok[2] = t2;
+  it.tok[3] = t3;
+  const bool ok = (magic == kPlanMagic) & (idx < n_items);
+  it.a = a;
+  it.r = r;
+  it.n_tok = ok ? n_tok : 0;
+  it.j0 = j0;
+  it.more = more;
+  it.base = (int64_t)(((uint64_t)(uint32_t)base_hi << 32) | (uint32_t)base_lo);
+  page0 = pg0;
+  page1 = pg1;
+}
+
+// a_loc entry `li` -> page id without a branch around the load: an out-of-range
+// index reads entry 0 and is rejected afterwards (n_loc > 0 is checked by the caller)
+__device__ __forceinline__ int64_t lookup_page_nobranch(const Tables& t, int64_t li, bool want) {
+  const bool in = want & ((uint64_t)li < (uint64_t)t.n_loc);
+  const int64_t page = t.a_loc[in ? li : 0];
+  return (in & ((uint64_t)page < (uint64_t)t.n_pages)) ? page : (int64_t)-1;
 }
 
 // ---------------------------------------------------------------------------
@@ -187,6 +212,85 @@ struct ShrinkArgs {
   unsigned long long* dbg;  // [grid][4] clock stamps: start, item known, weights arrived, end
 #endif
 };
+
+// The common case in straight-line code: hidden <= 4096 (one pass), all tokens
+// of the run fit the LDS staging area, no rows beyond the item.  Every global
+// load is unconditional (absent tokens / rows read a valid dummy address and are
+// discarded) so that no branch separates the loads: first the activations, then
+// both weight pages; the LDS stores wait for the activations only.
+template <typename T>
+__device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it, int proj, int r_eff,
+                                            const int64_t (&page)[2], u32x4* s_x) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nvec = p.h_in >> 3;
+  const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
+  const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
+
+  u32x4 xr[kTT][2];
+#pragma unroll
+  for (int t = 0; t < kTT; ++t) {
+    const int tk = t < it.n_tok ? it.tok[t] : it.tok[0];
+    const u32x4* xrow = xg + (int64_t)tk * nvec;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int v = i * 256 + tid;
+      xr[t][i] = xrow[v < nvec ? v : 0];
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);  // keep the activation loads in front: the LDS stores wait for them only
+  u32x4 wv[2][kVecPerPass];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const u32x4* src = reinterpret_cast<const u32x4*>(wbase + (page[i] >= 0 ? page[i] : 0) * p.page_elems);
+#pragma unroll
+    for (int c = 0; c < kVecPerPass; ++c) {
+      const int v = c * kWave + lane;
+      wv[i][c] = src[v < nvec ? v : 0];
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int t = 0; t < kTT; ++t)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int v = i * 256 + tid;
+      if (t < it.n_tok && v < nvec) s_x[t * nvec + v] = xr[t][i];
+    }
+  __syncthreads();
+
+  float acc[2][kTT];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int t = 0; t < kTT; ++t) acc[i][t] = 0.f;
+#pragma unroll
+  for (int t = 0; t < kTT; ++t) {
+    if (t < it.n_tok) {
+#pragma unroll
+      for (int c = 0; c < kVecPerPass; ++c) {
+        const int v = c * kWave + lane;
+        if (v < nvec) {
+          const u32x4 xv = s_x[t * nvec + v];
+#pragma unroll
+          for (int i = 0; i < 2; ++i) acc[i][t] = dot8<T>(wv[i][c], xv, acc[i][t]);
+        }
+      }
+    }
+  }
+  uint16_t* y = reinterpret_cast<uint16_t*>(p.y[proj]);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = it.j0 + wave + 4 * i;
+#pragma unroll
+    for (int t = 0; t < kTT; ++t) {
+      if (t < it.n_tok) {
+        const float sum = wave_sum(acc[i][t]);
+        if (lane == 0 && page[i] >= 0 && row < r_eff) y[(int64_t)it.tok[t] * p.y_cols + row] = T::from_float(sum);
+      }
+    }
+  }
+}
 
 // 4 wavefronts; wavefront w takes rows j0+w and j0+w+4 of one projection.  A
 // q/k/v call launches three workgroups per item (projection-major, so that with
@@ -208,9 +312,10 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   const int proj = blockIdx.x / p.units;
   const int unit = blockIdx.x - proj * p.units;
   Item it;
-  const int* rec = nullptr;
+  const int* rec = PLANNED ? p.plan + kPlanHeaderWords + (int64_t)unit * kItemWords : nullptr;
+  int plan_pg0 = -1, plan_pg1 = -1;
   if (PLANNED) {
-    rec = load_item(p.plan, unit, it);
+    load_item(p.plan, unit, p.qkvo0 + proj, wave, wave + 4, it, plan_pg0, plan_pg1);
   } else {
     const int b = unit / p.blocks;
     discover_run(p.t, p.batch, b, it);
@@ -223,11 +328,32 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
     p.dbg[(size_t)blockIdx.x * 4 + 3] = 0ull;
   }
 #endif
+  // page ids of this wavefront's two rows, read before any branch
+  int64_t page2[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int jr = wave + 4 * i;
+    if (PLANNED)
+      page2[i] = i == 0 ? plan_pg0 : plan_pg1;
+    else
+      page2[i] = lookup_page_nobranch(p.t, it.base + (int64_t)it.r * (p.qkvo0 + proj) + it.j0 + jr,
+                                      it.n_tok > 0 && p.t.n_loc > 0);
+  }
   if (it.n_tok <= 0) return;
   const int r_eff = it.r < p.y_cols ? it.r : p.y_cols;
   if (it.j0 >= r_eff) return;  // uniform over the workgroup
 
   const int nvec = p.h_in >> 3;
+  if (nvec <= 512 && it.n_tok <= p.lds_tt && !(PLANNED && it.more)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (it.j0 + wave + 4 * i >= r_eff) page2[i] = -1;
+    shrink_fast<T>(p, it, proj, r_eff, page2, s_x);
+#ifdef SLORA_TIMING
+    if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
+#endif
+    return;
+  }
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
   int row[NTASK];
   const u32x4* wrow[NTASK];
@@ -495,17 +621,17 @@ __device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, con
 // or -2 to look it up in a_loc.
 template <typename T>
 __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const Item& it, int r_eff, int kk,
-                                           int64_t page, float scale, bool vec_ok, uint16_t* s_strip) {
+                                           int64_t page, bool vec_ok, uint16_t* s_strip) {
   const int64_t base_li = it.base + (int64_t)it.r * (p.qkvo0 + proj);
   if (!vec_ok) {
-    expand_scalar<T>(p, proj, it, r_eff, kk, base_li, scale);
+    expand_scalar<T>(p, proj, it, r_eff, kk, base_li, load_scale(p.scales, p.scales_dtype, it.a));
     return;
   }
   if (page == -2) page = lookup_page(p.t, base_li + kk);
   if (page < 0) return;
   const uint16_t* wpage = reinterpret_cast<const uint16_t*>(p.w) + page * p.page_elems;
   const int64_t flat0 = (int64_t)kk * p.page_elems;
-  expand_page<T>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
+  expand_page<T>(p, proj, it, r_eff, wpage, flat0, load_scale(p.scales, p.scales_dtype, it.a), s_strip);
 }
 
 // Expand has nothing to share between wavefronts (the delta row is 16 bytes per
@@ -524,9 +650,9 @@ __global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p)
   const int jr = (sub & 1) * 4 + wave;  // page inside the item's block
 
   Item it;
-  const int* rec = nullptr;
+  int plan_pg = -1, plan_pg_unused = -1;
   if (PLANNED) {
-    rec = load_item(p.plan, unit, it);
+    load_item(p.plan, unit, p.qkvo0 + proj, jr, jr, it, plan_pg, plan_pg_unused);
   } else {
     const int b = unit / p.blocks;
     discover_run(p.t, p.batch, b, it);
@@ -549,18 +675,17 @@ __global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p)
   else
     extra = it.j0 + kRB >= p.blocks * kRB;
   if (k >= n_pg && !extra) return;
-  const float scale = load_scale(p.scales, p.scales_dtype, it.a);
   const bool pow2 = (r & (r - 1)) == 0;
   // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
   const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
                       (p.page_elems % (8 * r)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
   if (k < n_pg) {
-    const int64_t page = PLANNED ? (int64_t)rec[IT_PAGES + (p.qkvo0 + proj) * kRB + jr] : (int64_t)-2;
-    expand_one<T>(p, proj, it, r_eff, k, page, scale, vec_ok, s_strip);
+    const int64_t page = PLANNED ? (int64_t)plan_pg : (int64_t)-2;
+    expand_one<T>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
   }
   if (extra) {
 #pragma unroll 1
-    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, scale, vec_ok, s_strip);
+    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
   }
 }
 
