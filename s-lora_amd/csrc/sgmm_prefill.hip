@@ -49,6 +49,15 @@ __device__ __forceinline__ int64_t seg_page(const SegTables& t, int64_t li) {
   return (uint64_t)page < (uint64_t)t.n_pages ? page : -1;
 }
 
+// a_loc entry `li` -> page id with the load outside any branch: an unwanted or
+// out-of-range index reads entry 0 and is rejected afterwards.  Callers issue
+// several of these back to back so the loads overlap.
+__device__ __forceinline__ int64_t seg_page_nobranch(const SegTables& t, int64_t li, bool want) {
+  const bool in = want & ((uint64_t)li < (uint64_t)t.n_loc);
+  const int64_t page = t.a_loc[in ? li : 0];
+  return (in & ((uint64_t)page < (uint64_t)t.n_pages)) ? page : (int64_t)-1;
+}
+
 // Request `req`: its adapter, rank, first row and row count clipped to the
 // buffers.  False if the request has nothing to do.
 __device__ __forceinline__ bool seg_lookup(const SegTables& t, int req, int64_t& a, int& r, int& row0, int& rows) {
@@ -104,10 +113,63 @@ __device__ void shrink_generic(const SegShrinkArgs& p, int r_eff, int64_t base_l
   }
 }
 
+// One wavefront's share of the K loop of a 32-token x (16 * NT)-rank tile.  Its K
+// steps (32 k each) come in adjacent pairs -- global step (i / 2) * 16 + 2 * wave +
+// (i & 1) -- so the two halves of a 128-byte line are read back to back by the same
+// wavefront.  The loads of one step are in flight while the previous one is
+// multiplied; two workgroups share a compute unit (128 registers per lane), so one
+// can stream while the other looks up its pages or reduces its partial sums.  No load sits inside a branch (the wait
+// counters then stay exact): the main loop only runs where all of its steps exist,
+// and the tail re-reads the last step where one does not.
+template <typename T, int NT>
+__device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xrow)[2], const uint16_t* const (&wrow)[4],
+                                              int ksteps, int wave, int lg, int h_in, f32x4 (&acc)[2][4]) {
+  const int full = ksteps / (2 * kShrWaves), extra = ksteps - full * 2 * kShrWaves - 2 * wave;
+  const int n = 2 * full + (extra <= 0 ? 0 : (extra >= 2 ? 2 : 1));  // steps of this wavefront
+  if (n == 0) return;
+  const bool ragged_k = (h_in & 31) != 0;
+  auto load_step = [&](int i, u32x4 (&af)[2], u32x4 (&bf)[NT]) {
+    if (i >= n) i = n - 1;
+    int k = ((i >> 1) * (2 * kShrWaves) + 2 * wave + (i & 1)) * 32 + lg * 8;
+    const bool k_in = k < h_in;
+    if (!k_in) k = 0;
+#pragma unroll
+    for (int f = 0; f < 2; ++f) af[f] = ldg16(xrow[f] + k);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) bf[t] = ldg16(wrow[t] + k);
+    if (ragged_k && !k_in) {
+#pragma unroll
+      for (int f = 0; f < 2; ++f) af[f] = zero16();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) bf[t] = zero16();
+    }
+  };
+  auto mul_step = [&](const u32x4 (&af)[2], const u32x4 (&bf)[NT]) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int f = 0; f < 2; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
+  };
+  u32x4 a0[2], b0[NT], a1[2], b1[NT];
+  load_step(0, a0, b0);
+  int i = 0;
+  for (; i + 2 < n; i += 2) {
+    load_step(i + 1, a1, b1);
+    mul_step(a0, b0);
+    load_step(i + 2, a0, b0);
+    mul_step(a1, b1);
+  }
+  // one or two steps are left; step i is loaded
+  load_step(i + 1, a1, b1);
+  mul_step(a0, b0);
+  if (i + 1 < n) mul_step(a1, b1);
+}
+
 template <typename T>
-__global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrinkArgs p) {
+__global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // consecutive workgroup ids go to the 8 XCDs in turn: keep all token tiles of a
   // request on one XCD (request % 8) so its weight rows are fetched by one L2
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
@@ -145,16 +207,19 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrin
   for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
     const int nb_cnt = p.max_rank - nb0 < kShrNB ? p.max_rank - nb0 : kShrNB;
     if (nb0 < r_eff) {
-      // weight rows of the four B fragments
+      // weight rows of the four B fragments: the four page lookups go out together;
+      // a row that does not exist (j >= r_eff, bad page id) reads pool page 0 --
+      // its products only reach output columns that are zeroed below
       const uint16_t* wrow[4];
+      {
+        int64_t pg[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const int j = nb0 + t * 16 + lr;
-        wrow[t] = nullptr;
-        if (j < r_eff) {
-          const int64_t page = seg_page(p.t, base_li + j);
-          if (page >= 0) wrow[t] = wg + page * p.w_stride;
+        for (int t = 0; t < 4; ++t) {
+          const int j = nb0 + t * 16 + lr;
+          pg[t] = seg_page_nobranch(p.t, base_li + j, j < r_eff && p.t.n_loc > 0);
         }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) wrow[t] = wg + (pg[t] >= 0 ? pg[t] : 0) * p.w_stride;
       }
       const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
       f32x4 acc[2][4];
@@ -163,36 +228,11 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_shrink_kernel(const SegShrin
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-      // This wavefront's K steps are s = wave, wave + 8, ...  A three-stage register
-      // pipeline keeps the loads of two steps in flight while a third is multiplied.
-      const int my_steps = ksteps > wave ? (ksteps - wave + kShrWaves - 1) / kShrWaves : 0;
-      auto load_step = [&](int i, u32x4 (&af)[2], u32x4 (&bf)[4]) {
-        const int k = (wave + i * kShrWaves) * 32 + lg * 8;
-        const bool k_ok = i < my_steps && k < p.h_in;
-#pragma unroll
-        for (int f = 0; f < 2; ++f) af[f] = k_ok ? ldg16(xrow[f] + k) : zero16();
-#pragma unroll
-        for (int t = 0; t < 4; ++t) bf[t] = (k_ok && t < n_tiles && wrow[t] != nullptr) ? ldg16(wrow[t] + k) : zero16();
-      };
-      auto mul_step = [&](const u32x4 (&af)[2], const u32x4 (&bf)[4]) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          if (t < n_tiles) {
-#pragma unroll
-            for (int f = 0; f < 2; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
-          }
-        }
-      };
-      u32x4 a0[2], b0[4], a1[2], b1[4], a2[2], b2[4];
-      load_step(0, a0, b0);
-      load_step(1, a1, b1);
-      for (int i = 0; i < my_steps; i += 3) {
-        load_step(i + 2, a2, b2);
-        mul_step(a0, b0);
-        load_step(i + 3, a0, b0);
-        mul_step(a1, b1);
-        load_step(i + 4, a1, b1);
-        mul_step(a2, b2);
+      switch (n_tiles) {
+        case 1: shrink_k_loop<T, 1>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
+        case 2: shrink_k_loop<T, 2>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
+        case 3: shrink_k_loop<T, 3>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
+        default: shrink_k_loop<T, 4>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
       }
       // C tile: lane holds column lr, rows 4*lg + i
       float* mine = s_part + wave * (kShrTM * kShrLd);
@@ -292,28 +332,43 @@ __device__ __forceinline__ void expand_load(const SegExpandArgs& p, int r, int r
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
   const uint16_t* og = reinterpret_cast<const uint16_t*>(p.o);
   const uint32_t page_elems = (uint32_t)p.page_elems;
+  // phase 1: every page id (loads back to back, no branch in between)
+  int64_t page[4][KS];
+  uint32_t off[4][KS];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     const int n = nb + 32 * (t >> 1) + 8 * (lr >> 2) + 4 * (t & 1) + (lr & 3);
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d = s * 32 + lg * 8;
-      buf.a[t][s] = zero16();
-      if (live && n < p.feat_out && d < r_eff) {
-        const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
-        const uint32_t pg = flat / page_elems, off = flat - pg * page_elems;
-        const int64_t page = seg_page(p.t, base_li + pg);
-        if (page >= 0) buf.a[t][s] = ldg16(wg + page * p.w_stride + off);
-      }
+      const bool want = live && n < p.feat_out && d < r_eff && p.t.n_loc > 0;
+      const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
+      const uint32_t pg = flat / page_elems;
+      off[t][s] = flat - pg * page_elems;
+      page[t][s] = seg_page_nobranch(p.t, base_li + pg, want);
     }
   }
+  // phase 2: every fragment, from a valid dummy address where there is none
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const bool ok = page[t][s] >= 0;
+      buf.a[t][s] = ldg16(wg + (ok ? page[t][s] * p.w_stride + off[t][s] : 0));
+    }
 #pragma unroll
   for (int f = 0; f < kExpMF; ++f)
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int n = nb + 32 * h + 8 * lg;
-      buf.y[f][h] = (live && row_ok[f] && n < p.feat_out) ? ldg16(og + orow[f] + n) : zero16();
+      const bool ok = live && row_ok[f] && n < p.feat_out;
+      buf.y[f][h] = ldg16(og + orow[f] + (ok ? n : 0));  // a row that is not there repeats row 0 and is never stored
     }
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+      if (page[t][s] < 0) buf.a[t][s] = zero16();
 }
 
 template <typename T, int KS>
