@@ -26,6 +26,14 @@ for _p in (ROOT, os.path.join(ROOT, "s-lora_amd")):
 
 METRIC = "LoRA tokens/s + achieved HBM GB/s (% peak), S2 decode BGMV batch 256"
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, from rocprofv3 counter runs of this
+# file (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for
+# a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
+# None where not measured.
+TRAFFIC_BYTES = {
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80655596,  # 74364140 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70295448,     # the q/k/v launch
+}
 
 
 def parse_args():
@@ -35,7 +43,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--batch", type=int, default=256)
-    ap.add_argument("--workload", choices=["s2", "s4", "s6"], default="s2")
+    ap.add_argument("--workload", choices=["s2", "s4", "s6", "c3"], default="s2",
+                    help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels, "
+                         "reported in the same format with their own metric name")
     ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused"], default="planned-fused",
                     help="dropin: 8 stateless dispatch_bgmv calls per layer exactly as the reference issues them; "
                          "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer); "
@@ -70,11 +80,15 @@ class StepBuffers:
 
 
 def make_step(w, bufs, mode):
-    """Returns (step, shrink_sweep, expand_sweep, kernel-name suffix).  With a
-    planned mode the plan is rebuilt inside every step (one extra small launch,
-    as a caller would do once per decode step); its item count was read back
-    once when the plan was first made -- the synchronisation a caller pays per
-    step, like the reference's own ``.item()`` at lora_unordered_batch_infer.py:64."""
+    """Returns (step, families).  `families` maps a label to (sweep, kernel
+    name, launches per sweep, algorithmic bytes per launch): one sweep per kind
+    of launch the step issues, over all layers, so that each kind's launch
+    duration can be timed by itself.  With a planned mode the plan is rebuilt
+    inside every step (one extra small launch, as a caller would do once per
+    decode step); its item count was read back once when the plan was first
+    made -- the synchronisation a caller pays per step, like the reference's own
+    ``.item()`` at lora_unordered_batch_infer.py:64."""
+    import torch
     import slora_hip
     bgmv = slora_hip.dispatch_bgmv
     t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
@@ -82,39 +96,68 @@ def make_step(w, bufs, mode):
     fused = mode.endswith("fused")
     plan = slora_hip.make_plan(*t, w.max_rank, w.n_pages) if planned else None
     kw = {"plan": plan} if planned else {}
+    L = w.n_layers
+    ty = "F16" if w.dtype == torch.float16 else "BF16"
+    pl = "true" if planned else "false"
 
-    def shrink_sweep():
-        for l in range(w.n_layers):
-            for p in range(3):
-                bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
-            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling, **kw)
+    def qkv_shrink(l):
+        slora_hip.dispatch_bgmv_qkv_shrink(bufs.delta[0], bufs.delta[1], bufs.delta[2], bufs.x_in[l],
+                                           w.key_buffer[l], *t, **kw)
 
-    def expand_sweep():
-        for l in range(w.n_layers):
-            for p in range(3):
-                bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling, **kw)
-            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling, **kw)
+    def qkv_expand(l):
+        slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
+                                           bufs.delta[2], w.value_buffer[l], *t, w.a_scaling, **kw)
+
+    def shrink(l, p):
+        bgmv(bufs.delta[p % 3], bufs.x_in[l] if p < 3 else bufs.x_att[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
+
+    def expand(l, p):
+        bgmv(bufs.y[l][p], bufs.delta[p % 3], w.value_buffer[l], *t, p, w.a_scaling, **kw)
+
+    def over_layers(fn, *a):
+        def sweep():
+            for l in range(L):
+                fn(l, *a)
+        return sweep
+
+    def all_proj(fn):
+        def sweep():
+            for l in range(L):
+                for p in range(4):
+                    fn(l, p)
+        return sweep
+
+    sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
+    if fused:
+        families = {
+            "qkv_shrink": (over_layers(qkv_shrink), sk, L, w.qkv_shrink_bytes()),
+            "o_shrink": (over_layers(shrink, 3), sk, L, w.shrink_bytes()),
+            "qkv_expand": (over_layers(qkv_expand), ek % 3, L, w.qkv_expand_bytes()),
+            "o_expand": (over_layers(expand, 3), ek % 1, L, w.expand_bytes(w.h_out[3])),
+        }
+    else:
+        families = {
+            "shrink": (all_proj(shrink), sk, 4 * L, w.shrink_bytes()),
+            "expand": (all_proj(expand), ek % 1, 4 * L, sum(w.expand_bytes(h) for h in w.h_out) / 4),
+        }
 
     def step():
         if planned:
             slora_hip.rebuild_plan(plan, *t, w.n_pages)
-        for l in range(w.n_layers):
+        for l in range(L):
             if fused:
-                slora_hip.dispatch_bgmv_qkv_shrink(bufs.delta[0], bufs.delta[1], bufs.delta[2], bufs.x_in[l],
-                                                   w.key_buffer[l], *t, **kw)
-                slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0],
-                                                   bufs.delta[1], bufs.delta[2], w.value_buffer[l], *t, w.a_scaling,
-                                                   **kw)
+                qkv_shrink(l)
+                qkv_expand(l)
             else:
                 # call order of lora_unordered_batch_infer.py:254-318
                 for p in range(3):
-                    bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
-                    bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, p, w.a_scaling, **kw)
+                    shrink(l, p)
+                    expand(l, p)
             # o projection, lora_unordered_batch_infer.py:428-448
-            bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, 3, w.a_scaling, **kw)
-            bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, 3, w.a_scaling, **kw)
+            shrink(l, 3)
+            expand(l, 3)
 
-    return step, shrink_sweep, expand_sweep
+    return step, families
 
 
 def graphed(fn, torch):
@@ -224,6 +267,73 @@ def cpu_baseline(w, bufs, torch, reps_arg):
     }
 
 
+MFMA_PEAK_TFLOPS = 2500.0
+
+
+def main_prefill(args, torch, device):
+    """C3: q/k/v/o segmented shrink and expand over a prefill batch, per layer."""
+    import slora_hip
+    from slora_hip import workloads
+    L = min(args.layers, 4)
+    w, seg = workloads.c3_prefill(device, n_layers=L)
+    T, H, R = seg.n_tokens, w.hidden, w.max_rank
+    g = torch.Generator(device=device)
+    g.manual_seed(7)
+    x = [torch.randn((T, H), generator=g, device=device, dtype=torch.float32).to(w.dtype) for _ in range(L)]
+    y = [torch.zeros((T, H), device=device, dtype=w.dtype) for _ in range(L)]
+    d = torch.zeros((T, R), device=device, dtype=w.dtype)
+    t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
+
+    def shrink_sweep():
+        for l in range(L):
+            for p in range(4):
+                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len)
+
+    def expand_sweep():
+        for l in range(L):
+            for p in range(4):
+                slora_hip.lora_get_qkvo_fwd_expand(d, w.value_buffer[l].view(-1, H), y[l], w.a_scaling, *t, H, p, R,
+                                                   seg.max_len)
+
+    def step():
+        for l in range(L):
+            for p in range(4):
+                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len)
+                slora_hip.lora_get_qkvo_fwd_expand(d, w.value_buffer[l].view(-1, H), y[l], w.a_scaling, *t, H, p, R,
+                                                   seg.max_len)
+
+    use_graph = args.launch == "graph"
+    wrap = (lambda f: graphed(f, torch)) if use_graph else (lambda f: f)
+    reps = max(5, args.steps)
+    ms_step = time_region(wrap(step), reps, args.warmup, torch)
+    kernels = {}
+    flops = seg.flops(w, H)
+    for label, sweep, kname, nbytes in (
+            ("shrink", shrink_sweep, "sgmm_shrink_kernel<BF16>", seg.shrink_bytes(w)),
+            ("expand", expand_sweep, "sgmm_expand_kernel<BF16, 2>", seg.expand_bytes(w, H))):
+        us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
+        kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
+                          "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                          "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                          "TFLOPs": round(flops / us / 1e6, 1),
+                          "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
+    dom = max(kernels.values(), key=lambda k: k["us_per_launch"])
+    out = {
+        "metric": "LoRA prefill tokens/s + achieved HBM GB/s (% peak), C3 segmented shrink/expand",
+        "value": round(T / (ms_step * 1e-3 / L), 1),
+        "unit": "tokens/s per layer",
+        "n_gpus": 1, "steps": reps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "layers": L, "tokens": T, "requests": int(seg.lens_np.size),
+                   "launch": args.launch, "launches_per_step": 8 * L},
+        "roofline": {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": dom["frac"], "traffic": None,
+                     "algorithmic_bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"]},
+        "kernels": kernels,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -240,6 +350,9 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.workload == "c3":
+        main_prefill(args, torch, device)
+        return
     if args.workload == "s2":
         w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch)
     elif args.workload == "s4":
@@ -253,13 +366,13 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    step, shrink_sweep, expand_sweep = make_step(w, bufs, args.mode)
+    step, families = make_step(w, bufs, args.mode)
+    fused = args.mode.endswith("fused")
     if args.check:
         check_layer0(w, bufs, torch)
 
-    run_step, run_shrink, run_expand = step, shrink_sweep, expand_sweep
-    if args.launch == "graph":
-        run_step, run_shrink, run_expand = graphed(step, torch), graphed(shrink_sweep, torch), graphed(expand_sweep, torch)
+    use_graph = args.launch == "graph"
+    run_step = graphed(step, torch) if use_graph else step
 
     def time_steps(fn):
         """exactly K steps between two synchronisations; ms per step"""
@@ -283,26 +396,27 @@ def main():
         for m in ("dropin", "fused", "planned", "planned-fused"):
             if m == args.mode:
                 continue
-            st, _, _ = make_step(w, bufs, m)
-            fn = graphed(st, torch) if args.launch == "graph" else st
+            st, _ = make_step(w, bufs, m)
+            fn = graphed(st, torch) if use_graph else st
             ms = time_steps(fn)
             other_modes[m] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1),
                               "launches_per_step": w.n_layers * (4 if m.endswith("fused") else 8)}
 
-    # ---- per-kernel launch duration: sweeps of one kernel family, same stream ---------
-    n_launch = w.n_layers * 4
+    # ---- launch duration of every kind of launch in the step: a sweep of that kind over
+    # all layers, HIP events on the stream the kernels run on (back-to-back launches, so
+    # the figure includes the gap between two launches)
     reps = max(5, args.steps // 2)
-    shrink_us = time_region(run_shrink, reps, 3, torch) * 1e3 / n_launch
-    expand_us = time_region(run_expand, reps, 3, torch) * 1e3 / n_launch
-    shrink_bytes = sum(w.shrink_bytes() for _ in range(4)) / 4
-    expand_bytes = sum(w.expand_bytes(h) for h in w.h_out) / 4
-    shrink_gbs = shrink_bytes / (shrink_us * 1e-6) / 1e9
-    expand_gbs = expand_bytes / (expand_us * 1e-6) / 1e9
-    dominant = ("bgmv_expand_kernel", expand_us, expand_bytes, expand_gbs) if expand_us >= shrink_us else \
-               ("bgmv_shrink_kernel", shrink_us, shrink_bytes, shrink_gbs)
-    # the sweeps above launch the single-projection kernels (planned or stateless as the mode says)
+    kernels = {}
+    for label, (sweep, kname, n_launch, nbytes) in families.items():
+        fn = graphed(sweep, torch) if use_graph else sweep
+        us = time_region(fn, reps, 3, torch) * 1e3 / n_launch
+        gbs = nbytes / (us * 1e-6) / 1e9
+        kernels[label] = {"kernel": kname, "launches_per_step": n_launch, "us_per_launch": round(us, 3),
+                          "bytes_per_launch": int(nbytes), "GBps": round(gbs, 1),
+                          "frac": round(gbs / HBM_PEAK_GBS, 4)}
+    dom = max(kernels.values(), key=lambda k: k["us_per_launch"] * k["launches_per_step"])
 
-    step_gbs = w.step_bytes() / (ms_per_step * 1e-3) / 1e9
+    step_gbs = w.step_bytes(fused) / (ms_per_step * 1e-3) / 1e9
     out = {
         "metric": METRIC,
         "value": round(w.batch / (ms_per_step * 1e-3), 1),
@@ -324,31 +438,25 @@ def main():
             "pool_pages_per_layer": w.n_pages,
             "mode": args.mode,
             "launch": args.launch,
-            "launches_per_step": w.n_layers * (4 if args.mode.endswith("fused") else 8) +
-                                 (1 if args.mode.startswith("planned") else 0),
+            "launches_per_step": w.n_layers * (4 if fused else 8) + (1 if args.mode.startswith("planned") else 0),
         },
         "step_hbm": {
-            "algorithmic_bytes_per_step": w.step_bytes(),
+            "algorithmic_bytes_per_step": w.step_bytes(fused),
             "achieved_GBps": round(step_gbs, 1),
             "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
         },
         "roofline": {
-            "kernel": dominant[0],
+            "kernel": dom["kernel"],
             "bound": "hbm",
-            "achieved": round(dominant[3], 1),
+            "achieved": dom["GBps"],
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": round(dominant[3] / HBM_PEAK_GBS, 4),
-            "traffic": None,
-            "algorithmic_bytes_per_launch": int(dominant[2]),
-            "us_per_launch": round(dominant[1], 3),
+            "frac": dom["frac"],
+            "traffic": TRAFFIC_BYTES.get((args.workload, w.batch, args.mode, dom["kernel"])),
+            "algorithmic_bytes_per_launch": dom["bytes_per_launch"],
+            "us_per_launch": dom["us_per_launch"],
         },
-        "kernels": {
-            "bgmv_shrink_kernel": {"us_per_launch": round(shrink_us, 3), "bytes_per_launch": int(shrink_bytes),
-                                   "GBps": round(shrink_gbs, 1), "frac": round(shrink_gbs / HBM_PEAK_GBS, 4)},
-            "bgmv_expand_kernel": {"us_per_launch": round(expand_us, 3), "bytes_per_launch": int(expand_bytes),
-                                   "GBps": round(expand_gbs, 1), "frac": round(expand_gbs / HBM_PEAK_GBS, 4)},
-        },
+        "kernels": kernels,
     }
     if other_modes:
         out["modes"] = other_modes

@@ -70,11 +70,21 @@ class DecodeWorkload:
     def _index_bytes(self, u) -> int:
         return int(self.batch * 8 + u.size * (16 + 2) + self.ranks[u].sum() * 8)
 
-    def layer_bytes(self) -> int:
+    def qkv_shrink_bytes(self) -> int:
+        """One launch covering q, k and v: the three per-call figures with x read once."""
+        return 3 * self.shrink_bytes() - 2 * self.batch * self.hidden * 2
+
+    def qkv_expand_bytes(self) -> int:
+        return sum(self.expand_bytes(h) for h in self.h_out[:3])
+
+    def layer_bytes(self, fused: bool = False) -> int:
+        if fused:
+            return (self.qkv_shrink_bytes() + self.shrink_bytes() + self.qkv_expand_bytes() +
+                    self.expand_bytes(self.h_out[3]))
         return sum(self.shrink_bytes() + self.expand_bytes(h) for h in self.h_out)
 
-    def step_bytes(self) -> int:
-        return self.n_layers * self.layer_bytes()
+    def step_bytes(self, fused: bool = False) -> int:
+        return self.n_layers * self.layer_bytes(fused)
 
     def gathered_layer_bytes(self) -> int:
         """Same formulas with every token fetching its own copy of the weights."""
@@ -173,3 +183,54 @@ def s6_decode(device, n_layers=8, batch=1024, n_adapters=2000, n_pages=None, dty
                                  device, hidden=8192, n_layers=n_layers, n_adapters=n_adapters, rank_choices=[64],
                                  batch=batch, n_pages=n_pages, dtype=dtype, h_out=[8192, 1024, 1024, 8192],
                                  ids="uniform", heads=64, seed=seed, occupancy=0.0, fill_noise=False)
+
+
+# ---- prefill ------------------------------------------------------------------
+@dataclass
+class PrefillSegments:
+    """Requests of a prefill batch laid end to end: request i owns token rows
+    ``b_start_loc[i] + [0, b_seq_len[i])`` and uses adapter ``b_indicies[i]``."""
+    lens_np: np.ndarray
+    ids_np: np.ndarray
+    b_start_loc: torch.Tensor = None  # int32
+    b_seq_len: torch.Tensor = None    # int32
+    b_indicies: torch.Tensor = None   # int64
+
+    @property
+    def n_tokens(self) -> int:
+        return int(self.lens_np.sum())
+
+    @property
+    def max_len(self) -> int:
+        return int(self.lens_np.max())
+
+    # algorithmic bytes and flops of one call over pool workload ``w``
+    def shrink_bytes(self, w) -> int:
+        u = np.unique(self.ids_np)
+        return int(self.n_tokens * w.hidden * 2 + self.n_tokens * w.max_rank * 2 + w.ranks[u].sum() * w.hidden * 2)
+
+    def expand_bytes(self, w, h_out) -> int:
+        u = np.unique(self.ids_np)
+        return int(2 * self.n_tokens * h_out * 2 + self.n_tokens * w.max_rank * 2 + w.ranks[u].sum() * h_out * 2)
+
+    def flops(self, w, h) -> int:
+        return int(2 * h * (w.ranks[self.ids_np] * self.lens_np).sum())
+
+
+def c3_prefill(device, n_layers=4, n_pages=65536, seed=3):
+    """64 requests of 8..512 tokens sorted by adapter, 100 adapters of ranks
+    {64,32,16,8}, bfloat16, hidden 4096, pages scattered over the pool."""
+    w = build_decode_workload("C3 prefill: hidden 4096, 64 requests of 8..512 tokens, 100 adapters ranks {64,32,16,8}, bf16",
+                              device, hidden=4096, n_layers=n_layers, n_adapters=100, rank_choices=[64, 32, 16, 8],
+                              batch=1, n_pages=n_pages, dtype=torch.bfloat16, seed=seed)
+    rng = np.random.default_rng(seed)
+    n_req = 64
+    lens = rng.integers(8, 513, size=n_req).astype(np.int32)
+    ids = np.sort(rng.integers(0, 100, size=n_req)).astype(np.int64)
+    start = np.zeros(n_req, np.int32)
+    start[1:] = np.cumsum(lens)[:-1]
+    seg = PrefillSegments(lens_np=lens, ids_np=ids)
+    seg.b_start_loc = torch.from_numpy(start).to(device)
+    seg.b_seq_len = torch.from_numpy(lens).to(device)
+    seg.b_indicies = torch.from_numpy(ids).to(device)
+    return w, seg
