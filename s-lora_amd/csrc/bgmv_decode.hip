@@ -189,11 +189,12 @@ __device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx,
   page1 = pg1;
 }
 
-// a_loc entry `li` -> page id without a branch around the load: an out-of-range
-// index reads entry 0 and is rejected afterwards (n_loc > 0 is checked by the caller)
+// a_loc entry `li` -> page id without a branch around the load: an unwanted or
+// out-of-range index reads a_start[0] instead (the table has at least one adapter
+// whenever a kernel is launched) and is rejected afterwards
 __device__ __forceinline__ int64_t lookup_page_nobranch(const Tables& t, int64_t li, bool want) {
   const bool in = want & ((uint64_t)li < (uint64_t)t.n_loc);
-  const int64_t page = t.a_loc[in ? li : 0];
+  const int64_t page = *(in ? t.a_loc + li : t.a_start);
   return (in & ((uint64_t)page < (uint64_t)t.n_pages)) ? page : (int64_t)-1;
 }
 
@@ -882,6 +883,170 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
   }
 }
 
+// The same plan for batches of up to kFastPlanBatch tokens, built by several
+// workgroups.  Every workgroup derives the runs, their order and the queues by
+// itself, entirely in LDS (the work is small and identical everywhere, so no
+// exchange between workgroups is needed); the item records, which are most of the
+// bytes and carry the page lookups, are then shared out: 16 lanes write one record
+// as twelve 16-byte stores, eight of them holding four page ids each whose lookups
+// are in flight together.
+constexpr int kFastPlanBatch = 1024;
+
+__global__ __launch_bounds__(kPlanThreads) void bgmv_plan_fast_kernel(int* __restrict__ plan, Tables t, int batch,
+                                                                      int rank_cap, int max_items) {
+  __shared__ int s_bins[kFastPlanBatch];    // adapter of a token, -1: none
+  __shared__ int s_run[kFastPlanBatch];     // token -> run, valid at a run's first token
+  __shared__ int s_ra[kFastPlanBatch], s_rr[kFastPlanBatch], s_rn[kFastPlanBatch];  // run: adapter, rank, items
+  __shared__ int s_blo[kFastPlanBatch], s_bhi[kFastPlanBatch];                      // run: a_start of its adapter
+  __shared__ int s_ntok[kFastPlanBatch];
+  __shared__ int s_toks[kFastPlanBatch * kTT];
+  __shared__ int s_before[kFastPlanBatch + 1];  // sorted position -> items in front of the run there
+  __shared__ int s_order[kFastPlanBatch];       // sorted position -> run
+  __shared__ int s_wave[kPlanWaves];
+  __shared__ int s_max_rank, s_total;
+  __shared__ int s_qstart[kXcds], s_qlen[kXcds];
+  const int tid = threadIdx.x;
+  if (tid == 0) {
+    s_max_rank = 0;
+    s_total = 0;
+  }
+  if (tid < kXcds) {
+    s_qstart[tid] = 0x7fffffff;
+    s_qlen[tid] = 0;
+  }
+  // one token per thread (batch <= kPlanThreads == kFastPlanBatch)
+  int a = -1;
+  if (tid < batch) {
+    const int64_t a64 = t.bins[tid];
+    a = ((uint64_t)a64 < (uint64_t)t.n_adapters && a64 <= 0x7fffffffLL) ? (int)a64 : -1;
+  }
+  int64_t len = 0, base = 0;
+  if (a >= 0) {
+    len = t.a_len[a];
+    base = t.a_start[a];
+  }
+  s_bins[tid] = a;
+  s_ntok[tid] = 0;
+  __syncthreads();
+  // my number among the tokens of my adapter, and the first token of my group of kTT
+  int pos = 0, first = tid;
+  const int q_end = tid < batch ? tid : 0;
+  for (int q = 0; q < q_end; ++q) {
+    if (s_bins[q] == a) {
+      if (pos % kTT == 0) first = q;
+      ++pos;
+    }
+  }
+  if (pos % kTT == 0) first = tid;
+  const int r = (a >= 0 && len > 0) ? (int)(len >> 2) : 0;
+  const bool member = r > 0;
+  const bool leader = member && first == tid;
+  int n_runs = 0;
+  const int idx = block_exclusive_scan(leader ? 1 : 0, s_wave, &n_runs);
+  int n_it = 0;
+  if (leader) {
+    const int r_listed = r < rank_cap ? r : rank_cap;
+    n_it = (r_listed + kRB - 1) / kRB;
+    s_run[tid] = idx;
+    s_ra[idx] = a;
+    s_rr[idx] = r;
+    s_rn[idx] = n_it;
+    s_blo[idx] = (int)(uint32_t)(uint64_t)base;
+    s_bhi[idx] = (int)(uint32_t)((uint64_t)base >> 32);
+    atomicMax(&s_max_rank, r);
+    atomicAdd(&s_total, n_it);
+  }
+  __syncthreads();
+  if (member) {
+    const int run = s_run[first];
+    s_toks[run * kTT + pos % kTT] = tid;
+    atomicAdd(&s_ntok[run], 1);
+  }
+  const int total = s_total;
+  // order by (adapter, first token): items in front of my run, and runs in front of it
+  if (leader) {
+    int before = 0, rank_pos = 0;
+    for (int o = 0; o < n_runs; ++o) {
+      const int oa = s_ra[o];
+      if (oa < a || (oa == a && o < idx)) {  // runs are numbered in token order
+        before += s_rn[o];
+        ++rank_pos;
+      }
+    }
+    int q = (int)(((int64_t)before * kXcds) / (total > 0 ? total : 1));
+    if (q > kXcds - 1) q = kXcds - 1;
+    s_before[rank_pos] = before;
+    s_order[rank_pos] = idx;
+    atomicMin(&s_qstart[q], before);
+    atomicAdd(&s_qlen[q], n_it);
+  }
+  __syncthreads();
+  int max_len = 0;
+  for (int q = 0; q < kXcds; ++q) max_len = s_qlen[q] > max_len ? s_qlen[q] : max_len;
+  int n_items = kXcds * max_len;
+  if (n_items > max_items) n_items = 0;  // cannot happen with the capacity slora_bgmv_plan_bytes() reserves
+
+  // ---- records ----
+  const int sub = tid & 15;
+  const int n_groups = (int)gridDim.x * (kPlanThreads / 16);
+  for (int rec_i = (int)blockIdx.x * (kPlanThreads / 16) + (tid >> 4); rec_i < n_items; rec_i += n_groups) {
+    const int q = rec_i % kXcds, k = rec_i / kXcds;
+    const bool real = k < s_qlen[q];
+    int run = 0, i = 0;
+    if (real) {
+      const int srt = s_qstart[q] + k;  // index of the item in sorted order
+      int lo = 0, hi = n_runs;          // last sorted position whose `before` is <= srt
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (s_before[mid] <= srt) lo = mid; else hi = mid;
+      }
+      run = s_order[lo];
+      i = srt - s_before[lo];
+    }
+    const int ra = s_ra[run], rr = s_rr[run], rn = s_rn[run], n_tok = s_ntok[run];
+    const int64_t rbase = (int64_t)(((uint64_t)(uint32_t)s_bhi[run] << 32) | (uint32_t)s_blo[run]);
+    const int j0 = i * kRB;
+    int w0 = 0, w1 = 0, w2 = 0, w3 = 0;
+    if (sub >= 2 && sub < 10) {
+      const int proj = (sub - 2) >> 1, jr0 = ((sub - 2) & 1) * 4;
+      int64_t pg[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        pg[c] = lookup_page_nobranch(t, rbase + (int64_t)proj * rr + j0 + jr0 + c,
+                                     real && n_tok > 0 && j0 + jr0 + c < rr && t.n_loc > 0);
+      w0 = (pg[0] >= 0 && pg[0] <= 0x7fffffffLL) ? (int)pg[0] : -1;
+      w1 = (pg[1] >= 0 && pg[1] <= 0x7fffffffLL) ? (int)pg[1] : -1;
+      w2 = (pg[2] >= 0 && pg[2] <= 0x7fffffffLL) ? (int)pg[2] : -1;
+      w3 = (pg[3] >= 0 && pg[3] <= 0x7fffffffLL) ? (int)pg[3] : -1;
+    } else if (real) {
+      if (sub == 0) {
+        w0 = ra, w1 = rr, w2 = n_tok < kTT ? n_tok : kTT, w3 = j0;
+      } else if (sub == 1) {
+        w0 = n_tok > 0 ? s_toks[run * kTT + 0] : 0;
+        w1 = n_tok > 1 ? s_toks[run * kTT + 1] : 0;
+        w2 = n_tok > 2 ? s_toks[run * kTT + 2] : 0;
+        w3 = n_tok > 3 ? s_toks[run * kTT + 3] : 0;
+      } else if (sub == 10) {
+        w0 = s_blo[run], w1 = s_bhi[run];
+        w2 = (i == rn - 1 && rr > rank_cap) ? 1 : 0;
+      }
+    }
+    if (sub < 12) {
+      int4 v = make_int4(w0, w1, w2, w3);
+      *reinterpret_cast<int4*>(plan + kPlanHeaderWords + (int64_t)rec_i * kItemWords + sub * 4) = v;
+    }
+  }
+  if (blockIdx.x == 0 && tid == 0) {
+    plan[PH_MAGIC] = kPlanMagic;
+    plan[PH_NITEMS] = n_items;
+    plan[PH_MAXRANK] = s_max_rank;
+    plan[PH_BATCH] = batch;
+    plan[PH_TT] = kTT;
+    plan[PH_RANKCAP] = rank_cap;
+    plan[PH_NRUNS] = n_runs;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -973,6 +1138,8 @@ int shrink_common(const void* plan, int64_t n_items, int64_t rank_cap, void* con
   ShrinkArgs p{};
   int rc = fill_tables(p.t, tables, bins, n_pages);
   if (rc != SLORA_OK) return rc;
+  // no adapter or no adapter page: every lookup would be rejected
+  if (p.t.n_adapters == 0 || p.t.n_loc == 0) return SLORA_OK;
   if (x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
   for (int i = 0; i < nproj; ++i)
     if (y[i] == nullptr) return SLORA_ERR_NULL_POINTER;
@@ -1015,6 +1182,7 @@ int expand_common(const void* plan, int64_t n_items, int64_t rank_cap, void* con
   ExpandArgs p{};
   int rc = fill_tables(p.t, tables, bins, n_pages);
   if (rc != SLORA_OK) return rc;
+  if (p.t.n_adapters == 0 || p.t.n_loc == 0) return SLORA_OK;
   if (w == nullptr || scales == nullptr) return SLORA_ERR_NULL_POINTER;
   for (int i = 0; i < nproj; ++i)
     if (y[i] == nullptr || x[i] == nullptr) return SLORA_ERR_NULL_POINTER;
@@ -1118,6 +1286,14 @@ int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* ta
   if (rc != SLORA_OK) return rc;
   const int64_t max_items = plan_max_items(batch, rank_cap);
   if (max_items > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  if (batch <= kFastPlanBatch) {
+    int64_t grid = (max_items + kPlanThreads / 16 - 1) / (kPlanThreads / 16);
+    grid = grid < 1 ? 1 : (grid > 16 ? 16 : grid);
+    hipLaunchKernelGGL(bgmv_plan_fast_kernel, dim3((uint32_t)grid), dim3(kPlanThreads), 0,
+                       reinterpret_cast<hipStream_t>(stream), static_cast<int*>(plan), t, (int)batch, (int)rank_cap,
+                       (int)max_items);
+    return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+  }
   int* scratch = static_cast<int*>(plan) + kPlanHeaderWords + max_items * kItemWords;
   hipLaunchKernelGGL(bgmv_plan_kernel, dim3(1), dim3(kPlanThreads), 0, reinterpret_cast<hipStream_t>(stream),
                      static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items, scratch);

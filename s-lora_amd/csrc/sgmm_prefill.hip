@@ -50,11 +50,12 @@ __device__ __forceinline__ int64_t seg_page(const SegTables& t, int64_t li) {
 }
 
 // a_loc entry `li` -> page id with the load outside any branch: an unwanted or
-// out-of-range index reads entry 0 and is rejected afterwards.  Callers issue
-// several of these back to back so the loads overlap.
+// out-of-range index reads a_start[0] instead (there is at least one adapter
+// whenever a request reaches this point) and is rejected afterwards.  Callers
+// issue several of these back to back so the loads overlap.
 __device__ __forceinline__ int64_t seg_page_nobranch(const SegTables& t, int64_t li, bool want) {
   const bool in = want & ((uint64_t)li < (uint64_t)t.n_loc);
-  const int64_t page = t.a_loc[in ? li : 0];
+  const int64_t page = *(in ? t.a_loc + li : t.a_start);
   return (in & ((uint64_t)page < (uint64_t)t.n_pages)) ? page : (int64_t)-1;
 }
 
