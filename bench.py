@@ -144,6 +144,9 @@ def make_step(w, bufs, mode):
     def step():
         if planned:
             slora_hip.rebuild_plan(plan, *t, w.n_pages)
+        else:
+            # a new batch every step: calls that pass no plan may reuse one only within the step
+            slora_hip.clear_plan_cache()
         for l in range(L):
             if fused:
                 qkv_shrink(l)

@@ -9,6 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("SLORA_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libslora_hip.so")
 
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
+MAX_RANK = 512  # SLORA_MAX_RANK of include/slora_hip.h
 
 OK = 0
 ERR_NULL_POINTER, ERR_BAD_DTYPE, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_ALIGNMENT, ERR_LAUNCH = -1, -2, -3, -4, -5, -6

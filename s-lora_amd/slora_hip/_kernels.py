@@ -13,6 +13,8 @@ device fault here.
 from __future__ import annotations
 
 import ctypes as C
+import os
+import weakref
 
 import torch
 
@@ -127,6 +129,62 @@ def make_plan(start_indicies, lora_ranks, loc_indicies, indicies, rank_cap, n_pa
     return plan
 
 
+class _PlanCache:
+    """Plans built on behalf of callers that pass none.  The reference's engine
+    issues all 8 x n_layers ``dispatch_bgmv`` calls of a decode step with the same
+    four index tensors (lora_unordered_batch_infer.py:254-318, 428-448), so the
+    first call of a step builds the plan and the others reuse it.
+
+    An entry is reused only if the four tensors are the very same Python objects
+    (held through weak references) at the same ``_version`` (every in-place torch
+    operation raises it), on the same stream, for the same output width and pool
+    size.  Code that rewrites an index tensor behind torch's back (a raw pointer
+    handed to a custom kernel) must call ``clear_plan_cache()`` or set
+    ``SLORA_PLAN_CACHE=0``.  Nothing is cached while the stream is being captured
+    into a graph: a plan built there would not exist until the graph is replayed.
+    """
+
+    def __init__(self, capacity: int = 4):
+        self.capacity = capacity
+        self.entries = []
+        self.hits = 0
+        self.builds = 0
+
+    def clear(self) -> None:
+        self.entries.clear()
+
+    def get(self, tensors, rank_cap: int, n_pages: int, stream: int):
+        versions = tuple(t._version for t in tensors)
+        for i, (refs, vers, cap, pages, strm, plan) in enumerate(self.entries):
+            if cap == rank_cap and pages == n_pages and strm == stream and vers == versions and \
+                    all(r() is t for r, t in zip(refs, tensors)):
+                if i:
+                    self.entries.insert(0, self.entries.pop(i))
+                self.hits += 1
+                return plan
+        plan = make_plan(*tensors, rank_cap, n_pages, readback=True)
+        self.builds += 1
+        self.entries.insert(0, (tuple(weakref.ref(t) for t in tensors), versions, rank_cap, n_pages, stream, plan))
+        del self.entries[self.capacity:]
+        return plan
+
+
+_plan_cache = _PlanCache()
+
+
+def clear_plan_cache() -> None:
+    """Forget every plan built for calls that passed none."""
+    _plan_cache.clear()
+
+
+def _auto_plan(start_indicies, lora_ranks, loc_indicies, indicies, rank_cap: int, n_pages: int, stream: int):
+    if os.environ.get("SLORA_PLAN_CACHE", "1") == "0" or indicies.numel() == 0:
+        return None
+    if rank_cap <= 0 or rank_cap > _cabi.MAX_RANK or torch.cuda.is_current_stream_capturing():
+        return None
+    return _plan_cache.get((start_indicies, lora_ranks, loc_indicies, indicies), int(rank_cap), int(n_pages), stream)
+
+
 def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales, plan=None) -> None:
     """``y`` (in place) from ``x`` and the paged adapter pool ``w``.
 
@@ -139,6 +197,8 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
 
     ``plan`` (keyword, optional, not in the reference): a ``BgmvPlan`` from
     ``make_plan`` for this batch; same results, fewer dependent table reads.
+    Without it the plan of the last call with the same index tensors is reused
+    (see ``_PlanCache``); ``plan=False`` forces the kernels that need no plan.
     """
     _check_input(y, "y")
     _check_input(x, "x")
@@ -161,6 +221,11 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     page_elems = w.size(1) * w.size(2)
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
     code = _DTYPE_CODE[x.dtype]
+    stream = _stream(x)
+    if plan is None:
+        plan = _auto_plan(start_indicies, lora_ranks, loc_indicies, indicies, min(h_in, h_out), w.size(0), stream)
+    elif plan is False:
+        plan = None
     if plan is not None and plan.batch != batch:
         raise RuntimeError(f"plan was built for {plan.batch} tokens, this call has {batch}")
     if h_in < h_out:
@@ -169,20 +234,20 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
                                                None, x.data_ptr(), None, None, w.data_ptr(), C.byref(tables),
                                                indicies.data_ptr(), lora_scales.data_ptr(),
                                                _DTYPE_CODE[lora_scales.dtype], batch, h_in, h_out, 0, 0, page_elems,
-                                               w.size(0), qkvo, code, _stream(x))
+                                               w.size(0), qkvo, code, stream)
         else:
             rc = lib.slora_bgmv_expand(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables),
                                        indicies.data_ptr(), lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype],
-                                       batch, h_in, h_out, page_elems, w.size(0), qkvo, code, _stream(x))
+                                       batch, h_in, h_out, page_elems, w.size(0), qkvo, code, stream)
     else:
         if plan is not None:
             rc = lib.slora_bgmv_shrink_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 1, y.data_ptr(), None,
                                                None, x.data_ptr(), w.data_ptr(), C.byref(tables), indicies.data_ptr(),
-                                               batch, h_in, h_out, page_elems, w.size(0), qkvo, code, _stream(x))
+                                               batch, h_in, h_out, page_elems, w.size(0), qkvo, code, stream)
         else:
             rc = lib.slora_bgmv_shrink(y.data_ptr(), x.data_ptr(), w.data_ptr(), C.byref(tables),
                                        indicies.data_ptr(), batch, h_in, h_out, page_elems, w.size(0), qkvo, code,
-                                       _stream(x))
+                                       stream)
     if rc == _cabi.ERR_UNSUPPORTED:
         raise RuntimeError(no_kernel)
     _cabi.check(rc, "dispatch_bgmv", f"(h_in={h_in} h_out={h_out} qkvo={qkvo})")
@@ -207,6 +272,10 @@ def dispatch_bgmv_qkv_shrink(y_q, y_k, y_v, x, w, start_indicies, lora_ranks, lo
         raise RuntimeError(no_kernel)
     lib = _cabi.load_library()
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
+    if plan is None:
+        plan = _auto_plan(start_indicies, lora_ranks, loc_indicies, indicies, y_cols, w.size(0), _stream(x))
+    elif plan is False:
+        plan = None
     if plan is not None:
         rc = lib.slora_bgmv_shrink_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 3, y_q.data_ptr(),
                                            y_k.data_ptr(), y_v.data_ptr(), x.data_ptr(), w.data_ptr(),
@@ -244,6 +313,10 @@ def dispatch_bgmv_qkv_expand(y_q, y_k, y_v, x_q, x_k, x_v, w, start_indicies, lo
         raise RuntimeError(no_kernel)
     lib = _cabi.load_library()
     tables = _tables(start_indicies, lora_ranks, loc_indicies)
+    if plan is None:
+        plan = _auto_plan(start_indicies, lora_ranks, loc_indicies, indicies, x_cols, w.size(0), _stream(x_q))
+    elif plan is False:
+        plan = None
     if plan is not None:
         rc = lib.slora_bgmv_expand_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, 3, y_q.data_ptr(),
                                            y_k.data_ptr(), y_v.data_ptr(), x_q.data_ptr(), x_k.data_ptr(),

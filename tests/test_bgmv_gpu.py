@@ -18,6 +18,18 @@ RTOL, ATOL = 1e-2, 1e-3
 TDT = {"f16": torch.float16, "bf16": torch.bfloat16}
 
 
+@pytest.fixture(autouse=True, params=["cache", "stateless"])
+def plan_cache_mode(request, monkeypatch):
+    """Every test runs twice: with calls that pass no plan served by the
+    automatic plan cache (the default), and with the cache off, which sends the
+    same calls to the kernels that find their runs by themselves."""
+    import slora_hip
+    monkeypatch.setenv("SLORA_PLAN_CACHE", "1" if request.param == "cache" else "0")
+    slora_hip.clear_plan_cache()
+    yield request.param
+    slora_hip.clear_plan_cache()
+
+
 def dev(a, dtype, device):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device=device, dtype=dtype)
 
@@ -331,14 +343,14 @@ def test_planned_calls_equal_stateless_calls(gpu, dtype, hidden, ranks, batch, h
         d_s = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(4)]
         d_p = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(4)]
         for p in range(4):
-            dispatch_bgmv(d_s[p], g.x, g.key, *t, p, g.scales)
+            dispatch_bgmv(d_s[p], g.x, g.key, *t, p, g.scales, plan=False)
             dispatch_bgmv(d_p[p], g.x, g.key, *t, p, g.scales, plan=readback)
             assert torch.equal(d_s[p], d_p[p]), p
         y0 = [torch.randn((batch, c.h_out[p]), dtype=g.tdt, device=gpu) for p in range(4)]
         y_s = [v.clone() for v in y0]
         y_p = [v.clone() for v in y0]
         for p in range(4):
-            dispatch_bgmv(y_s[p], d_s[p], g.value, *t, p, g.scales)
+            dispatch_bgmv(y_s[p], d_s[p], g.value, *t, p, g.scales, plan=False)
             dispatch_bgmv(y_p[p], d_s[p], g.value, *t, p, g.scales, plan=readback)
             assert torch.equal(y_s[p], y_p[p]), p
         # fused q/k/v with a plan
@@ -348,6 +360,46 @@ def test_planned_calls_equal_stateless_calls(gpu, dtype, hidden, ranks, batch, h
         dispatch_bgmv_qkv_expand(y_f[0], y_f[1], y_f[2], d_f[0], d_f[1], d_f[2], g.value, *t, g.scales, plan=readback)
         for p in range(3):
             assert torch.equal(d_f[p], d_s[p]) and torch.equal(y_f[p], y_s[p]), p
+
+
+def test_automatic_plan_cache_follows_the_index_tensors(gpu, plan_cache_mode):
+    """Calls without a plan reuse one built at the first call for the same index
+    tensors; an in-place change of a tensor or a new tensor object rebuilds it,
+    and the results always equal those of the plan-free kernels."""
+    from slora_hip import dispatch_bgmv, _kernels
+    if plan_cache_mode != "cache":
+        pytest.skip("cache switched off")
+    c = make_case(77, 512, [16, 8, 32], 40, dtype="f16")
+    g = GpuCase(c, gpu)
+    cache = _kernels._plan_cache
+    cache.hits = cache.builds = 0
+
+    def both(bins):
+        t = (g.a_start, g.a_len, g.a_loc, bins)
+        d0 = torch.zeros((c.batch, 32), dtype=g.tdt, device=gpu)
+        d1 = torch.zeros_like(d0)
+        dispatch_bgmv(d0, g.x, g.key, *t, 1, g.scales, plan=False)
+        dispatch_bgmv(d1, g.x, g.key, *t, 1, g.scales)
+        assert torch.equal(d0, d1)
+        y0 = torch.zeros((c.batch, 512), dtype=g.tdt, device=gpu)
+        y1 = torch.zeros_like(y0)
+        dispatch_bgmv(y0, d0, g.value, *t, 1, g.scales, plan=False)
+        dispatch_bgmv(y1, d0, g.value, *t, 1, g.scales)
+        assert torch.equal(y0, y1)
+
+    both(g.bins)
+    assert (cache.builds, cache.hits) == (1, 1)   # shrink built it, expand reused it
+    both(g.bins)
+    assert (cache.builds, cache.hits) == (1, 3)
+    g.bins.copy_(torch.flip(g.bins, dims=[0]))     # new batch written in place: version changes
+    both(g.bins)
+    assert cache.builds == 2
+    both(g.bins.clone())                           # same contents in a new tensor object
+    assert cache.builds == 3
+    torch.cuda.synchronize()
+    with torch.cuda.stream(torch.cuda.Stream()):   # another stream never sees this stream's plan
+        both(g.bins)
+    assert cache.builds == 4
 
 
 def test_plan_is_rejected_for_another_batch_size(gpu):
