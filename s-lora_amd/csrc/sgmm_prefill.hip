@@ -12,6 +12,9 @@
 
 #include "common.hpp"
 #include "cabi_util.hpp"
+#ifdef SLORA_TIMING_PREFILL
+#include <stdlib.h>
+#endif
 
 namespace slora {
 namespace {
@@ -84,11 +87,15 @@ struct SegShrinkArgs {
   int64_t x_stride, w_stride, o_stride;  // elements per row
   int h_in, max_rank, qkvo, m_tiles;
   int vec_ok;  // every row start is 16-byte aligned and h_in % 8 == 0
+#ifdef SLORA_TIMING_PREFILL
+  unsigned long long* dbg;  // [grid][4] clock stamps: start, requests described, first tile done, end
+#endif
 };
 
 constexpr int kShrThreads = 512;
 constexpr int kShrWaves = kShrThreads / kWave;  // K is split over the 8 wavefronts
-constexpr int kShrTM = 32;                      // token rows per workgroup
+constexpr int kShrMF = 4;                       // 16-row A fragments per tile
+constexpr int kShrTM = 16 * kShrMF;             // token rows per tile
 constexpr int kShrNB = 64;                      // rank columns per pass
 constexpr int kShrLd = kShrNB + 4;              // LDS row pitch (floats) -> conflict-free C-tile stores
 
@@ -123,35 +130,35 @@ __device__ void shrink_generic(const SegShrinkArgs& p, int r_eff, int64_t base_l
 // counters then stay exact): the main loop only runs where all of its steps exist,
 // and the tail re-reads the last step where one does not.
 template <typename T, int NT>
-__device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xrow)[2], const uint16_t* const (&wrow)[4],
-                                              int ksteps, int wave, int lg, int h_in, f32x4 (&acc)[2][4]) {
+__device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xrow)[kShrMF], const uint16_t* const (&wrow)[4],
+                                              int ksteps, int wave, int lg, int h_in, f32x4 (&acc)[kShrMF][4]) {
   const int full = ksteps / (2 * kShrWaves), extra = ksteps - full * 2 * kShrWaves - 2 * wave;
   const int n = 2 * full + (extra <= 0 ? 0 : (extra >= 2 ? 2 : 1));  // steps of this wavefront
   if (n == 0) return;
   const bool ragged_k = (h_in & 31) != 0;
-  auto load_step = [&](int i, u32x4 (&af)[2], u32x4 (&bf)[NT]) {
+  auto load_step = [&](int i, u32x4 (&af)[kShrMF], u32x4 (&bf)[NT]) {
     if (i >= n) i = n - 1;
     int k = ((i >> 1) * (2 * kShrWaves) + 2 * wave + (i & 1)) * 32 + lg * 8;
     const bool k_in = k < h_in;
     if (!k_in) k = 0;
 #pragma unroll
-    for (int f = 0; f < 2; ++f) af[f] = ldg16(xrow[f] + k);
+    for (int f = 0; f < kShrMF; ++f) af[f] = ldg16(xrow[f] + k);
 #pragma unroll
     for (int t = 0; t < NT; ++t) bf[t] = ldg16(wrow[t] + k);
     if (ragged_k && !k_in) {
 #pragma unroll
-      for (int f = 0; f < 2; ++f) af[f] = zero16();
+      for (int f = 0; f < kShrMF; ++f) af[f] = zero16();
 #pragma unroll
       for (int t = 0; t < NT; ++t) bf[t] = zero16();
     }
   };
-  auto mul_step = [&](const u32x4 (&af)[2], const u32x4 (&bf)[NT]) {
+  auto mul_step = [&](const u32x4 (&af)[kShrMF], const u32x4 (&bf)[NT]) {
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int f = 0; f < 2; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
+      for (int f = 0; f < kShrMF; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
   };
-  u32x4 a0[2], b0[NT], a1[2], b1[NT];
+  u32x4 a0[kShrMF], b0[NT], a1[kShrMF], b1[NT];
   load_step(0, a0, b0);
   int i = 0;
   for (; i + 2 < n; i += 2) {
@@ -166,29 +173,14 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xrow)[2], 
   if (i + 1 < n) mul_step(a1, b1);
 }
 
+// One tile: token rows row_first .. row_first + m_cnt (m_cnt <= kShrTM) of a request
+// whose weight rows start at a_loc[base_li].  All threads of the workgroup call it
+// together; it ends with a barrier.
 template <typename T>
-__global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegShrinkArgs p) {
-  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
+__device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_part, int64_t row_first, int m_cnt,
+                                            int r_eff, int64_t base_li) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // consecutive workgroup ids go to the 8 XCDs in turn: keep all token tiles of a
-  // request on one XCD (request % 8) so its weight rows are fetched by one L2
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int req = (slot / p.m_tiles) * 8 + xcd;
-  const int m0 = (slot - (slot / p.m_tiles) * p.m_tiles) * kShrTM;
-  if (req >= p.t.n_requests) return;
-  int64_t a;
-  int r, row0, rows;
-  if (!seg_lookup(p.t, req, a, r, row0, rows)) return;
-  if (m0 >= rows) return;
-  const int m_cnt = rows - m0 < kShrTM ? rows - m0 : kShrTM;
-  const int r_eff = r < p.max_rank ? r : p.max_rank;
-  const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
-  if (!p.vec_ok) {
-    shrink_generic<T>(p, r_eff, base_li, row0, m0, m_cnt);
-    return;
-  }
-
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
   uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
@@ -197,12 +189,12 @@ __global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegSh
 
   // token rows of the two A fragments (clamped; rows past the end contribute
   // nothing because their results are never stored)
-  const uint16_t* xrow[2];
+  const uint16_t* xrow[kShrMF];
 #pragma unroll
-  for (int f = 0; f < 2; ++f) {
+  for (int f = 0; f < kShrMF; ++f) {
     int m = f * 16 + lr;
     if (m >= m_cnt) m = m_cnt - 1;
-    xrow[f] = xg + (int64_t)(row0 + m0 + m) * p.x_stride;
+    xrow[f] = xg + (row_first + m) * p.x_stride;
   }
 
   for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
@@ -223,9 +215,9 @@ __global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegSh
         for (int t = 0; t < 4; ++t) wrow[t] = wg + (pg[t] >= 0 ? pg[t] : 0) * p.w_stride;
       }
       const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
-      f32x4 acc[2][4];
+      f32x4 acc[kShrMF][4];
 #pragma unroll
-      for (int f = 0; f < 2; ++f)
+      for (int f = 0; f < kShrMF; ++f)
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -238,7 +230,7 @@ __global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegSh
       // C tile: lane holds column lr, rows 4*lg + i
       float* mine = s_part + wave * (kShrTM * kShrLd);
 #pragma unroll
-      for (int f = 0; f < 2; ++f)
+      for (int f = 0; f < kShrMF; ++f)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -253,11 +245,179 @@ __global__ __launch_bounds__(kShrThreads, 4) void sgmm_shrink_kernel(const SegSh
 #pragma unroll
           for (int wv = 0; wv < kShrWaves; ++wv) v += s_part[wv * (kShrTM * kShrLd) + m * kShrLd + c];
         }
-        og[(int64_t)(row0 + m0 + m) * p.o_stride + nb0 + c] = T::from_float(v);
+        og[(row_first + m) * p.o_stride + nb0 + c] = T::from_float(v);
       }
     }
     __syncthreads();
   }
+}
+
+// 16 token rows: the unit work is shared out in
+constexpr int kShrUnit = 16;
+constexpr int kShrMaxGrid = 256;  // one workgroup per compute unit
+constexpr int kShrChunk = 256;    // requests described at a time (keeps two workgroups' LDS within a compute unit)
+
+// inclusive prefix sum of `v` over the workgroup; *total receives the sum
+__device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave, int64_t* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int64_t inc = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int64_t up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  if (lane == kWave - 1) s_wave[wave] = inc;
+  __syncthreads();
+  int64_t before = 0, tot = 0;
+#pragma unroll
+  for (int wv = 0; wv < kShrWaves; ++wv) {
+    const int64_t c = s_wave[wv];
+    if (wv < wave) before += c;
+    tot += c;
+  }
+  __syncthreads();
+  *total = tot;
+  return before + inc;
+}
+
+// The requests are cut into units of 16 token rows, a unit of a rank-r request
+// costing kShrTM + r: its share of the bytes a full tile moves -- 16 activation
+// rows and a quarter of the r weight rows (a weight row measures as costly as an
+// activation row).  Laid end to end in request order, the units' cost line is
+// cut into gridDim.x equal parts, XCD-major: consecutive workgroup ids go to the
+// 8 XCDs in turn, so workgroup id -> part (id % 8) * (gridDim.x / 8) + id / 8
+// gives every XCD one contiguous eighth (neighbouring tiles of a request, which
+// read the same weight rows, share an L2) and every workgroup the same cost,
+// whatever the mix of request lengths and ranks.  A workgroup owns the units
+// whose start falls into its part and walks them as tiles of up to kShrMF units.
+template <typename T>
+__global__ __launch_bounds__(kShrThreads, 2) void sgmm_shrink_kernel(const SegShrinkArgs p) {
+  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
+  __shared__ int64_t s_wave[kShrWaves];
+  __shared__ int s_row0[kShrChunk], s_rows[kShrChunk], s_ub[kShrChunk], s_ue[kShrChunk], s_rank[kShrChunk];
+  __shared__ int64_t s_base[kShrChunk];
+  __shared__ int s_first, s_last;
+  const int tid = threadIdx.x;
+  const int parts = (int)gridDim.x;
+  const int part = (int)(blockIdx.x & 7) * (parts >> 3) + (int)(blockIdx.x >> 3);
+  const int row_cap = p.m_tiles * kShrTM;  // rows of a request past max_input_len are not touched
+#ifdef SLORA_TIMING_PREFILL
+  if (tid == 0) {
+    p.dbg[(size_t)blockIdx.x * 4 + 0] = __builtin_amdgcn_s_memrealtime();
+    p.dbg[(size_t)blockIdx.x * 4 + 2] = 0ull;
+  }
+#endif
+
+  // request -> cost of one of its units (0: nothing to do).  The loads sit outside
+  // every branch, in two dependent groups: (adapter id, first row, row count), then
+  // that adapter's (length, start) -- an invalid request re-reads entry 0.
+  auto describe = [&](int req, int64_t& base_li, int& r, int& row0, int& rows, int& units) -> int64_t {
+    const bool mine = tid < kShrChunk && req < p.t.n_requests;
+    const int rq = mine ? req : 0;
+    const int64_t a = p.t.b_indicies[rq];
+    row0 = p.t.b_start_loc[rq];
+    rows = p.t.b_seq_len[rq];
+    const bool a_ok = (uint64_t)a < (uint64_t)p.t.n_adapters;
+    const int64_t len = p.t.a_len[a_ok ? a : 0];
+    const int64_t start = p.t.a_start[a_ok ? a : 0];
+    r = (int)(len >> 2);
+    units = 0;
+    if (!mine || !a_ok || row0 < 0 || rows <= 0 || row0 >= p.t.n_tokens) return 0;
+    if (rows > p.t.n_tokens - row0) rows = p.t.n_tokens - row0;
+    if (rows > row_cap) rows = row_cap;
+    base_li = start + (int64_t)r * p.qkvo;
+    units = (rows + kShrUnit - 1) / kShrUnit;
+    return kShrTM + (r < p.max_rank ? r : p.max_rank);
+  };
+
+  // total cost (one pass when the requests fit one thread each)
+  int64_t total = 0;
+  if (p.t.n_requests > kShrChunk) {
+    for (int c0 = 0; c0 < p.t.n_requests; c0 += kShrChunk) {
+      int64_t base_li = 0;
+      int r = 0, row0 = 0, rows = 0, units = 0;
+      const int64_t cu = describe(c0 + tid, base_li, r, row0, rows, units);
+      int64_t tot = 0;
+      shrink_block_scan(cu * units, s_wave, &tot);
+      total += tot;
+    }
+  }
+  int64_t carry = 0;  // cost in front of the current chunk of requests
+  for (int c0 = 0; c0 < p.t.n_requests; c0 += kShrChunk) {
+    int64_t base_li = 0;
+    int r = 0, row0 = 0, rows = 0, units = 0;
+    const int64_t cu = describe(c0 + tid, base_li, r, row0, rows, units);
+    int64_t tot = 0;
+    const int64_t cp = carry + shrink_block_scan(cu * units, s_wave, &tot) - cu * units;  // cost in front of me
+    if (p.t.n_requests <= kShrChunk) total = tot;
+    if (total <= 0) return;
+    const int64_t lo = total * part / parts, hi = total * (part + 1) / parts;
+    // units of my request whose start cost cp + u * cu lies in [lo, hi)
+    int ub = 0, ue = 0;
+    if (units > 0) {
+      const int64_t b = lo > cp ? (lo - cp + cu - 1) / cu : 0;
+      const int64_t e = hi > cp ? (hi - cp + cu - 1) / cu : 0;
+      ub = b < units ? (int)b : units;
+      ue = e < units ? (int)e : units;
+    }
+    if (tid == 0) {
+      s_first = kShrChunk;
+      s_last = -1;
+    }
+    __syncthreads();
+    if (tid < kShrChunk) {
+      s_ub[tid] = ub;
+      s_ue[tid] = ue;
+      s_row0[tid] = row0;
+      s_rows[tid] = rows;
+      s_rank[tid] = r;
+      s_base[tid] = base_li;
+      if (ue > ub) {
+        atomicMin(&s_first, tid);
+        atomicMax(&s_last, tid);
+      }
+    }
+    __syncthreads();
+    // everything read back from LDS is the same in every lane: say so, so that the
+    // tile code keeps it in scalar registers and branches on it uniformly
+    auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+    const int first = uni(s_first), last = uni(s_last);
+#ifdef SLORA_TIMING_PREFILL
+    if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 1] = __builtin_amdgcn_s_memrealtime();
+#endif
+    for (int j = first; j <= last; ++j) {
+      const int u0 = uni(s_ub[j]), u1 = uni(s_ue[j]);
+      const int rj = uni(s_rank[j]);
+      const int r_eff = rj < p.max_rank ? rj : p.max_rank;
+      const int rw0 = uni(s_row0[j]), rows = uni(s_rows[j]);
+      const int64_t bl = s_base[j];
+      const int64_t base_li =
+          (int64_t)(((uint64_t)(uint32_t)uni((int)((uint64_t)bl >> 32)) << 32) | (uint32_t)uni((int)(uint32_t)bl));
+      for (int u = u0; u < u1; u += kShrMF) {
+        const int m0 = u * kShrUnit;
+        int m_end = (u + kShrMF < u1 ? u + kShrMF : u1) * kShrUnit;
+        if (m_end > rows) m_end = rows;
+        if (m_end <= m0) continue;
+        if (!p.vec_ok) {
+          shrink_generic<T>(p, r_eff, base_li, rw0, m0, m_end - m0);
+          __syncthreads();
+        } else {
+#ifndef SLORA_PROBE_SKIP_TILE
+          shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li);
+#endif
+#ifdef SLORA_TIMING_PREFILL
+          if (tid == 0 && p.dbg[(size_t)blockIdx.x * 4 + 2] == 0ull)
+            p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
+#endif
+        }
+      }
+    }
+    carry += tot;
+    __syncthreads();  // the tables are rewritten by the next chunk
+  }
+#ifdef SLORA_TIMING_PREFILL
+  if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -518,9 +678,13 @@ int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
     }
     attr_done = true;
   }
-  const int64_t grid = (int64_t)((p.t.n_requests + 7) / 8) * 8 * p.m_tiles;
+  // one workgroup per tile of token rows, at most kShrMaxGrid, a multiple of 8
+  int64_t tiles = ((int64_t)p.t.n_tokens + kShrTM - 1) / kShrTM + p.t.n_requests;
+  const int64_t by_len = (int64_t)p.t.n_requests * p.m_tiles;
+  if (by_len < tiles) tiles = by_len;
+  int64_t grid = (tiles + 7) / 8 * 8;
+  if (grid > kShrMaxGrid) grid = kShrMaxGrid;
   if (grid <= 0) return SLORA_OK;
-  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
@@ -557,6 +721,7 @@ int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables*
   SegShrinkArgs p{};
   int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
   if (rc != SLORA_OK) return rc;
+  if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
   if (o == nullptr || x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
   if (h_in == 0 || h_in > (1 << 21) || max_rank > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
   p.o = o;
@@ -570,6 +735,9 @@ int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables*
   p.qkvo = qkvo;
   p.m_tiles = (int)((max_input_len + kShrTM - 1) / kShrTM);
   p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
+#ifdef SLORA_TIMING_PREFILL
+  p.dbg = reinterpret_cast<unsigned long long*>(strtoull(getenv("SLORA_TIMING_BUF"), nullptr, 0));
+#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, s) : launch_seg_shrink<BF16>(p, s);
 }
@@ -593,6 +761,7 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
   SegExpandArgs p{};
   int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
   if (rc != SLORA_OK) return rc;
+  if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
   if (o == nullptr || x == nullptr || w == nullptr || scales == nullptr) return SLORA_ERR_NULL_POINTER;
   if (feat_out > (1 << 21) || max_rank > SLORA_MAX_RANK || page_elems > (1LL << 30)) return SLORA_ERR_UNSUPPORTED;
   p.o = o;

@@ -66,6 +66,16 @@ def test_prefill_chain_matches_oracle(gpu, dtype, hidden, ranks, n_req, lo, hi):
         check(c, g, p, R, gpu, seed=p)
 
 
+@pytest.mark.parametrize("n_req,lo,hi", [(257, 1, 9), (300, 1, 40), (700, 1, 6), (64, 60, 70)])
+def test_prefill_many_requests(gpu, n_req, lo, hi):
+    """More requests than the shrink kernel describes at a time (256), unsorted
+    adapters, request lengths around the unit (16) and tile (64) sizes."""
+    c = seg_case(500 + n_req, 256, [8, 16, 32, 64, 24], n_req, lo, hi, "bf16", sort=False)
+    g = GpuCase(c, gpu)
+    for p in (0, 3):
+        check(c, g, p, 64, gpu, seed=p)
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_prefill_gather_bit_exact(gpu, dtype):
     rng = np.random.default_rng(5)
