@@ -352,6 +352,12 @@ def main():
     slora_hip.load_library()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.calibrate_copy:
+        src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device=device)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     if args.workload == "c3":
         main_prefill(args, torch, device)
@@ -363,12 +369,6 @@ def main():
     else:
         w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024)
     bufs = StepBuffers(w, device)
-    if args.calibrate_copy:
-        src = torch.ones(128 * 1024 * 1024, dtype=torch.float16, device=device)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
     step, families = make_step(w, bufs, args.mode)
     fused = args.mode.endswith("fused")
     if args.check:
