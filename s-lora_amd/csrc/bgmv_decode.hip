@@ -26,9 +26,6 @@
 
 #include "common.hpp"
 #include "cabi_util.hpp"
-#ifdef SLORA_TIMING
-#include <stdlib.h>
-#endif
 
 namespace slora {
 namespace {
@@ -209,9 +206,6 @@ struct ShrinkArgs {
   Tables t;
   int64_t page_elems;
   int batch, h_in, y_cols, qkvo0, blocks, lds_tt, units;
-#ifdef SLORA_TIMING
-  unsigned long long* dbg;  // [grid][4] clock stamps: start, item known, weights arrived, end
-#endif
 };
 
 // The common case in straight-line code: hidden <= 4096 (one pass), all tokens
@@ -306,9 +300,6 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];   // [lds_tt][h_in / 8]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#ifdef SLORA_TIMING
-  const unsigned long long ts0 = __builtin_amdgcn_s_memrealtime();
-#endif
 
   const int proj = blockIdx.x / p.units;
   const int unit = blockIdx.x - proj * p.units;
@@ -322,13 +313,6 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
     discover_run(p.t, p.batch, b, it);
     it.j0 = (unit - b * p.blocks) * kRB;
   }
-#ifdef SLORA_TIMING
-  if (tid == 0) {
-    p.dbg[(size_t)blockIdx.x * 4 + 0] = ts0;
-    p.dbg[(size_t)blockIdx.x * 4 + 1] = it.n_tok > 0 ? __builtin_amdgcn_s_memrealtime() : 0ull;
-    p.dbg[(size_t)blockIdx.x * 4 + 3] = 0ull;
-  }
-#endif
   // page ids of this wavefront's two rows, read before any branch
   int64_t page2[2];
 #pragma unroll
@@ -350,9 +334,6 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
     for (int i = 0; i < 2; ++i)
       if (it.j0 + wave + 4 * i >= r_eff) page2[i] = -1;
     shrink_fast<T>(p, it, proj, r_eff, page2, s_x);
-#ifdef SLORA_TIMING
-    if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
-#endif
     return;
   }
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
@@ -420,9 +401,6 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
 
     for (int jb = it.j0; jb < j_end; jb += kRB) {
       if (jb != it.j0 || t0 != 0) open_block(jb, jb == it.j0);
-#ifdef SLORA_TIMING
-      if (tid == 0 && wv[0][0][0] != 0x12345678u) p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
-#endif
       float acc[NTASK][kTT];
 #pragma unroll
       for (int i = 0; i < NTASK; ++i)
@@ -467,9 +445,6 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
       }
     }
   }
-#ifdef SLORA_TIMING
-  if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -1157,9 +1132,6 @@ int shrink_common(const void* plan, int64_t n_items, int64_t rank_cap, void* con
   p.y_cols = (int)y_cols;
   p.qkvo0 = qkvo0;
   p.blocks = (int)((y_cols + kRB - 1) / kRB);
-#ifdef SLORA_TIMING
-  p.dbg = reinterpret_cast<unsigned long long*>(strtoull(getenv("SLORA_TIMING_BUF"), nullptr, 0));
-#endif
   const bool planned = plan != nullptr;
   const int64_t grid = planned ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);

@@ -77,17 +77,6 @@ __device__ __forceinline__ float dot8(u32x4 w, u32x4 x, float acc) {
   return acc;
 }
 
-// acc += sum_i f32(w_i) * xs[i] with xs already in float
-template <typename T>
-__device__ __forceinline__ float dot8f(u32x4 w, const float (&xs)[8], float acc) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    acc = __builtin_fmaf(T::lo(w[i]), xs[2 * i], acc);
-    acc = __builtin_fmaf(T::hi(w[i]), xs[2 * i + 1], acc);
-  }
-  return acc;
-}
-
 // ---- cross-lane sums -------------------------------------------------------
 // DPP controls: quad_perm(a,b,c,d) = a | b<<2 | c<<4 | d<<6; 0x141 = row_half_mirror,
 // 0x140 = row_mirror.  After xor-1 and xor-2 every quad is uniform, so the two
@@ -120,68 +109,6 @@ __device__ __forceinline__ float wave_sum(float v) {
   float c = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
   float d = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
   return (a + b) + (c + d);
-}
-
-// ---- tokens that share an adapter -----------------------------------------
-// A workgroup is launched for every token b.  Tokens with the same adapter
-// are processed together so the adapter's pages are read once: the tokens
-// whose bins equal `a` are numbered in order, cut into runs of `tt`, and the
-// first token of each run ("leader") does the run's work.  Returns the number
-// of tokens in b's run if b leads it (their indices in s_members[0..n)), else
-// 0.  Must be called by all NT threads of the block; s_masks holds NT/64
-// words.  The caller synchronises before reading s_members.
-template <int NT>
-__device__ __forceinline__ int find_run(const int64_t* __restrict__ bins, int64_t batch, int b, int64_t a,
-                                        int tt, uint64_t* s_masks, int* s_members) {
-  constexpr int NW = NT / kWave;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int total = 0;   // matches in chunks already processed
-  int pos_b = -1;  // b's number among the matches, once known
-  for (int64_t base = 0; base < batch; base += NT) {
-    const int64_t t = base + tid;
-    const bool m = t < batch && bins[t] == a;
-    const uint64_t ballot = __ballot(m);
-    if (base != 0) __syncthreads();  // previous chunk's masks fully consumed
-    if (lane == 0) s_masks[wave] = ballot;
-    __syncthreads();
-    int pre = total, chunk_total = 0, pre_b = total;
-    const int bw = (int)((b - base) >> 6), bl = (int)((b - base) & 63);
-    const bool b_here = b >= base && b < base + NT;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-      const uint64_t mk = s_masks[w];
-      const int pc = __popcll(mk);
-      if (w < wave) pre += pc;
-      if (b_here) {
-        if (w < bw) pre_b += pc;
-        if (w == bw) pre_b += __popcll(mk & ((1ull << bl) - 1ull));
-      }
-      chunk_total += pc;
-    }
-    pre += __popcll(ballot & ((1ull << lane) - 1ull));
-    if (b_here) {
-      pos_b = pre_b;
-      if (pos_b % tt != 0) return 0;  // uniform: every thread computed the same pos_b
-    }
-    if (pos_b >= 0 && m) {
-      const int k = pre - pos_b;
-      if (k >= 0 && k < tt) s_members[k] = (int)t;
-    }
-    total += chunk_total;
-    if (pos_b >= 0 && total - pos_b >= tt) break;
-  }
-  const int n = total - pos_b;
-  return n < tt ? n : tt;
-}
-
-// blockIdx -> (token, block-within-token).  Consecutive workgroup ids go to
-// the 8 XCDs in turn, each with its own L2; this mapping keeps all blocks of
-// one token on one XCD so its activations and tables are fetched by one L2.
-__device__ __forceinline__ void map_block(uint32_t id, uint32_t blocks_per_token, int& token, int& blk) {
-  const uint32_t xcd = id & 7u, slot = id >> 3;
-  const uint32_t grp = slot / blocks_per_token;
-  blk = (int)(slot - grp * blocks_per_token);
-  token = (int)(grp * 8u + xcd);
 }
 
 }  // namespace slora
