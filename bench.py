@@ -43,9 +43,10 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--batch", type=int, default=256)
-    ap.add_argument("--workload", choices=["s2", "s4", "s6", "c3"], default="s2",
-                    help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels, "
-                         "reported in the same format with their own metric name")
+    ap.add_argument("--workload", choices=["s2", "s4", "s6", "c3", "load"], default="s2",
+                    help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels; "
+                         "load: copying adapters into the pool; the last two are reported in the same format with "
+                         "their own metric names")
     ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused"], default="planned-fused",
                     help="dropin: 8 stateless dispatch_bgmv calls per layer exactly as the reference issues them; "
                          "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer); "
@@ -337,6 +338,51 @@ def main_prefill(args, torch, device):
     print(json.dumps(out), flush=True)
 
 
+def main_load(args, torch, device):
+    """Loading rank-64 adapters into the pools of 32 layers: for every adapter one
+    call scatters its 256 rows of 8 KiB into the key and value buffer of every
+    layer (64 buffers), as InferAdapter.load_lora_A/B do with 64 index_puts."""
+    import numpy as np
+    from slora_hip.infer_adapter import load_rows_into_pool
+    L, H, r, n_pages, n_adapters = min(args.layers, 32), 4096, 64, 16384, 8
+    bufs = [torch.zeros((n_pages, 32, H // 32), dtype=torch.float16, device=device) for _ in range(2 * L)]
+    rows = [[torch.randn((4 * r, 32, H // 32), device=device, dtype=torch.float32).to(torch.float16)
+             for _ in range(2 * L)] for _ in range(n_adapters)]
+    perm = np.random.default_rng(0).permutation(n_pages)
+    locs = [torch.from_numpy(perm[i * 4 * r:(i + 1) * 4 * r].astype(np.int64)).to(device) for i in range(n_adapters)]
+
+    def step():
+        for a in range(n_adapters):
+            load_rows_into_pool(bufs, rows[a], locs[a])
+
+    def torch_step():
+        for a in range(n_adapters):
+            for b in range(2 * L):
+                bufs[b][locs[a]] = rows[a][b]
+
+    use_graph = args.launch == "graph"
+    ms = time_region(graphed(step, torch) if use_graph else step, max(5, args.steps), args.warmup, torch)
+    ms_torch = time_region(graphed(torch_step, torch) if use_graph else torch_step, max(5, args.steps), args.warmup,
+                           torch)
+    nbytes = 2 * (4 * r) * H * 2 * 2 * L  # read + write per adapter
+    us = ms * 1e3 / n_adapters
+    gbs = nbytes / us / 1e3
+    out = {
+        "metric": "adapter load into the unified pool, GB/s moved (read + write)",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": max(5, args.steps), "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"{n_adapters} adapters of rank {r}, hidden {H}, {L} layers, key + value buffers",
+                   "launch": args.launch, "launches_per_step": n_adapters},
+        "roofline": {"kernel": "pool_scatter_kernel", "bound": "hbm", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": nbytes, "us_per_launch": round(us, 3)},
+        "torch_index_put": {"us_per_adapter": round(ms_torch * 1e3 / n_adapters, 3),
+                            "launches_per_adapter": 2 * L},
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -361,6 +407,9 @@ def main():
 
     if args.workload == "c3":
         main_prefill(args, torch, device)
+        return
+    if args.workload == "load":
+        main_load(args, torch, device)
         return
     if args.workload == "s2":
         w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch)

@@ -185,6 +185,49 @@ SLORA_API int slora_sgmm_expand(void* o, const void* x, const void* w, const slo
                       int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
                       int dtype, void* stream);
 
+/* ---- moving adapters in and out of the pool --------------------------------- */
+
+/* pool[loc[i]] = rows[i], i < n_rows, for n_bufs pool buffers in one go.
+ * Replaces the per-layer index_put of the adapter loader,
+ * `key_buffer[l][loc] = w_combined[0]` and `value_buffer[l][loc] = w_combined[1]`
+ * (slora/server/router/model_infer/infer_adapter.py:56-57, 81-82).
+ * dst_bufs / src_bufs are HOST arrays of n_bufs device pointers (e.g. the
+ * key_buffer and value_buffer of every layer, and the two halves of every
+ * layer's w_combined): src_bufs[b] holds n_rows rows of row_bytes bytes at
+ * src_row_stride_bytes, dst_bufs[b] holds n_pages pages at
+ * dst_row_stride_bytes.  loc is a device array of n_rows page ids shared by all
+ * buffers; a page id outside [0, n_pages) is skipped.  Duplicate page ids give
+ * an unspecified winner, as with index_put. */
+SLORA_API int slora_pool_scatter_rows(void* const* dst_bufs, const void* const* src_bufs, int n_bufs,
+                            const int64_t* loc, int64_t n_rows, int64_t row_bytes, int64_t dst_row_stride_bytes,
+                            int64_t src_row_stride_bytes, int64_t n_pages, void* stream);
+
+/* new_a_loc[new_a_start[i] + k] = old_a_loc[old_a_start[i] + k], k < old_a_len[i],
+ * i < n_adapters.  Replaces launch_var_len_copy_triton
+ * (slora/server/router/model_infer/infer_adapter.py:261-280); copies exactly
+ * old_a_len[i] entries (the reference's mask over-copies lists longer than its
+ * block of 256 into the next adapter's range).  A list that does not fit its
+ * table (n_old_loc / n_new_loc entries) is skipped. */
+SLORA_API int slora_var_len_copy(const int64_t* old_a_start, const int64_t* old_a_len, const int64_t* old_a_loc,
+                       const int64_t* new_a_start, int64_t* new_a_loc, int64_t n_adapters, int64_t n_old_loc,
+                       int64_t n_new_loc, void* stream);
+
+/* The index tables after dropping the adapters with keep[i] == 0, in one launch.
+ * Replaces the table rebuild of InferAdapter.offload_adapters
+ * (slora/server/router/model_infer/infer_adapter.py:186-258: a_len[left_ind],
+ * cumsum, a_scaling[left_ind], var_len_copy, torch.cat of the removed lists).
+ * Kept adapters keep their order; new_a_start is the running sum of their
+ * lengths; new_a_loc holds their page lists back to back; removed_pages holds the
+ * page lists of the dropped adapters back to back, in order (what goes back to
+ * the allocator).  counts[0..3] = kept adapters, kept page ids, dropped adapters,
+ * dropped page ids.  Output arrays must have room for the worst case
+ * (n_adapters / n_loc entries); work is n_adapters int64 of scratch owned by the
+ * caller.  a_scaling / new_a_scaling are scales_dtype (2 or 4 bytes per entry). */
+SLORA_API int slora_tables_compact(const slora_tables* tables, const void* a_scaling, int scales_dtype,
+                         const uint8_t* keep, int64_t* new_a_start, int64_t* new_a_len, int64_t* new_a_loc,
+                         void* new_a_scaling, int64_t* removed_pages, int64_t* counts, int64_t* work,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

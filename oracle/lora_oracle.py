@@ -328,6 +328,33 @@ def ref_var_len_copy(old_a_start, old_a_len, old_a_loc, new_a_start, new_size: i
     return out
 
 
+def ref_offload_tables(a_start, a_len, a_loc, a_scaling, keep):
+    """The table rebuild of ``InferAdapter.offload_adapters``
+    (infer_adapter.py:206-258) with ``keep[i]`` standing for "adapter i is in
+    reserve_adapter_dirs or carries the current prefetch tag" (:207-215).
+
+    Returns ``(new_a_start, new_a_len, new_a_loc, new_a_scaling, remove_ind)``:
+    ``new_a_len = a_len[left_ind]`` (:238), ``new_a_start`` its exclusive running
+    sum (:239-240), ``new_a_scaling = a_scaling[left_ind]`` (:241), ``new_a_loc``
+    the kept lists copied by var_len_copy (:243-244), ``remove_ind`` the removed
+    adapters' lists concatenated in order (:210, :224), which is what goes to
+    ``mem_manager.free``."""
+    a_start = np.asarray(a_start, dtype=np.int64)
+    a_len = np.asarray(a_len, dtype=np.int64)
+    a_loc = np.asarray(a_loc, dtype=np.int64)
+    left = [i for i in range(len(a_len)) if keep[i]]
+    gone = [i for i in range(len(a_len)) if not keep[i]]
+    new_len = a_len[left] if left else np.zeros(0, np.int64)
+    new_start = np.zeros(len(left), dtype=np.int64)
+    if len(left) > 1:
+        new_start[1:] = np.cumsum(new_len)[:-1]
+    new_loc = ref_var_len_copy(a_start[left], new_len, a_loc, new_start, int(new_len.sum())) if left else \
+        np.zeros(0, np.int64)
+    removed = [a_loc[int(a_start[i]): int(a_start[i]) + int(a_len[i])] for i in gone]
+    removed = np.concatenate(removed) if removed else np.zeros(0, np.int64)
+    return new_start, new_len, new_loc, np.asarray(a_scaling)[left], removed
+
+
 # ----------------------------------------------------------------------------
 # the reference's torch path on host cores (CPU baseline of the benchmark)
 # ----------------------------------------------------------------------------

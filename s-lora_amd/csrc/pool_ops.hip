@@ -1,0 +1,287 @@
+// Moving adapters in and out of the unified paged pool: the producers of every
+// byte the LoRA kernels read.
+//
+//   slora_pool_scatter_rows   pool[loc[i]] = rows[i] for several pool buffers at once
+//                             (slora/server/router/model_infer/infer_adapter.py:56-57,
+//                             81-82: `key_buffer[l][loc] = w_combined[0]`, one
+//                             index_put per layer and side in the reference)
+//   slora_var_len_copy        new_loc[new_start[i] + k] = old_loc[old_start[i] + k]
+//                             (infer_adapter.py:261-280, launch_var_len_copy_triton)
+//   slora_tables_compact      the index tables after some adapters are dropped, and the
+//                             page ids they give back (infer_adapter.py:186-258)
+//
+// All three are plain byte/integer movement, bound by HBM bandwidth (the first)
+// or by a handful of dependent round trips (the other two).
+
+#include "common.hpp"
+#include "cabi_util.hpp"
+
+namespace slora {
+namespace {
+
+// ---------------------------------------------------------------------------
+// scatter rows into pool pages
+// ---------------------------------------------------------------------------
+constexpr int kScatterBufs = 64;  // pool buffers served by one launch (pointers travel as kernel arguments)
+
+struct ScatterArgs {
+  void* dst[kScatterBufs];
+  const void* src[kScatterBufs];
+  const int64_t* loc;
+  int64_t n_rows, n_pages;
+  int64_t row_bytes, dst_stride, src_stride;  // bytes
+  int n_bufs;
+  int vec_ok;  // rows, strides and bases are multiples of 16 bytes
+};
+
+// One workgroup per (row, buffer): buffer-fastest, so the few workgroups that
+// read the same loc entry run together.  A row of 8 KiB is two 16-byte loads and
+// stores per lane, all loads issued before the stores.
+__global__ __launch_bounds__(256) void pool_scatter_kernel(const ScatterArgs p) {
+  const int64_t row = blockIdx.x / p.n_bufs;
+  const int buf = (int)(blockIdx.x - row * p.n_bufs);
+  const int64_t page = p.loc[row];
+  if ((uint64_t)page >= (uint64_t)p.n_pages) return;  // a page id outside the pool is skipped, not written
+  const char* s = static_cast<const char*>(p.src[buf]) + row * p.src_stride;
+  char* d = static_cast<char*>(p.dst[buf]) + page * p.dst_stride;
+  if (p.vec_ok) {
+    const int64_t nvec = p.row_bytes >> 4;
+    for (int64_t v0 = 0; v0 < nvec; v0 += 4 * 256) {
+      u32x4 t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t v = v0 + u * 256 + threadIdx.x;
+        t[u] = ldg16(s + ((v < nvec ? v : 0) << 4));
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t v = v0 + u * 256 + threadIdx.x;
+        if (v < nvec) *reinterpret_cast<u32x4*>(d + (v << 4)) = t[u];
+      }
+    }
+  } else {
+    for (int64_t b = threadIdx.x; b < p.row_bytes; b += 256) d[b] = s[b];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// variable-length copy of page-id lists
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void var_len_copy_kernel(const int64_t* __restrict__ old_start,
+                                                           const int64_t* __restrict__ len,
+                                                           const int64_t* __restrict__ old_loc,
+                                                           const int64_t* __restrict__ new_start,
+                                                           int64_t* __restrict__ new_loc, int64_t n_old_loc,
+                                                           int64_t n_new_loc) {
+  const int64_t i = blockIdx.x;
+  const int64_t n = len[i], os = old_start[i], ns = new_start[i];
+  if (n <= 0 || os < 0 || ns < 0 || os > n_old_loc - n || ns > n_new_loc - n) return;  // a list outside its table is skipped
+  for (int64_t k = threadIdx.x; k < n; k += 256) new_loc[ns + k] = old_loc[os + k];
+}
+
+// ---------------------------------------------------------------------------
+// table compaction
+// ---------------------------------------------------------------------------
+constexpr int kCompactThreads = 1024;
+constexpr int kCompactWaves = kCompactThreads / kWave;
+
+// inclusive prefix sums of two values over the workgroup, totals returned through tot_*
+__device__ __forceinline__ void compact_scan2(int64_t& a, int64_t& b, int64_t* s_a, int64_t* s_b, int64_t& tot_a,
+                                              int64_t& tot_b) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int64_t ua = __shfl_up(a, o, kWave), ub = __shfl_up(b, o, kWave);
+    if (lane >= o) {
+      a += ua;
+      b += ub;
+    }
+  }
+  if (lane == kWave - 1) {
+    s_a[wave] = a;
+    s_b[wave] = b;
+  }
+  __syncthreads();
+  int64_t ba = 0, bb = 0;
+  tot_a = 0;
+  tot_b = 0;
+  for (int wv = 0; wv < kCompactWaves; ++wv) {
+    if (wv < wave) {
+      ba += s_a[wv];
+      bb += s_b[wv];
+    }
+    tot_a += s_a[wv];
+    tot_b += s_b[wv];
+  }
+  __syncthreads();
+  a += ba;
+  b += bb;
+}
+
+struct CompactArgs {
+  const int64_t* a_start;
+  const int64_t* a_len;
+  const int64_t* a_loc;
+  const void* a_scaling;
+  const uint8_t* keep;
+  int64_t* new_start;
+  int64_t* new_len;
+  int64_t* new_loc;
+  void* new_scaling;
+  int64_t* removed;
+  int64_t* counts;  // [4]: kept adapters, kept page ids, dropped adapters, dropped page ids
+  int64_t* work;    // [n_adapters] destination offset of every adapter's list
+  int64_t n_adapters, n_loc;
+  int scale_bytes;
+};
+
+// One workgroup.  Pass 1 (a thread per adapter, 1024 at a time with running
+// totals): kept adapters are numbered in order and get the running sum of kept
+// lengths as their new start; dropped adapters get their offset in the list of
+// returned page ids.  Pass 2 (a wavefront per adapter): the lists are copied,
+// lanes over consecutive entries.
+__global__ __launch_bounds__(kCompactThreads) void tables_compact_kernel(const CompactArgs p) {
+  __shared__ int64_t s_a[kCompactWaves], s_b[kCompactWaves];
+  const int tid = threadIdx.x;
+  int64_t kept = 0, kept_loc = 0, dropped = 0, dropped_loc = 0;
+  for (int64_t i0 = 0; i0 < p.n_adapters; i0 += kCompactThreads) {
+    const int64_t i = i0 + tid;
+    const bool in = i < p.n_adapters;
+    int64_t len = in ? p.a_len[i] : 0;
+    const int64_t start = in ? p.a_start[i] : 0;
+    const bool k = in && p.keep[i] != 0;
+    if (len < 0 || start < 0 || start > p.n_loc - len) len = 0;  // a list outside a_loc counts as empty
+    // kept: (count, length) ; dropped: (count, length) -- two scans
+    int64_t kc = k ? 1 : 0, kl = k ? len : 0, tkc, tkl;
+    compact_scan2(kc, kl, s_a, s_b, tkc, tkl);
+    int64_t dc = (in && !k) ? 1 : 0, dl = (in && !k) ? len : 0, tdc, tdl;
+    compact_scan2(dc, dl, s_a, s_b, tdc, tdl);
+    if (in) {
+      if (k) {
+        const int64_t idx = kept + kc - 1, off = kept_loc + kl - len;
+        p.new_start[idx] = off;
+        p.new_len[idx] = len;
+        if (p.scale_bytes == 2)
+          static_cast<uint16_t*>(p.new_scaling)[idx] = static_cast<const uint16_t*>(p.a_scaling)[i];
+        else
+          static_cast<uint32_t*>(p.new_scaling)[idx] = static_cast<const uint32_t*>(p.a_scaling)[i];
+        p.work[i] = off;
+      } else {
+        p.work[i] = dropped_loc + dl - len;
+      }
+    }
+    kept += tkc;
+    kept_loc += tkl;
+    dropped += tdc;
+    dropped_loc += tdl;
+  }
+  if (tid == 0) {
+    p.counts[0] = kept;
+    p.counts[1] = kept_loc;
+    p.counts[2] = dropped;
+    p.counts[3] = dropped_loc;
+  }
+  __threadfence_block();
+  __syncthreads();  // work[] written above is read by other wavefronts below
+  const int lane = tid & 63, wave = tid >> 6;
+  for (int64_t i = wave; i < p.n_adapters; i += kCompactWaves) {
+    int64_t len = p.a_len[i];
+    const int64_t start = p.a_start[i];
+    if (len < 0 || start < 0 || start > p.n_loc - len) len = 0;
+    int64_t* dst = (p.keep[i] != 0 ? p.new_loc : p.removed) + p.work[i];
+    for (int64_t e = lane; e < len; e += kWave) dst[e] = p.a_loc[start + e];
+  }
+}
+
+}  // namespace
+}  // namespace slora
+
+extern "C" {
+
+int slora_pool_scatter_rows(void* const* dst_bufs, const void* const* src_bufs, int n_bufs, const int64_t* loc,
+                            int64_t n_rows, int64_t row_bytes, int64_t dst_row_stride_bytes,
+                            int64_t src_row_stride_bytes, int64_t n_pages, void* stream) {
+  using namespace slora;
+  if (n_bufs < 0 || n_rows < 0 || row_bytes < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (dst_row_stride_bytes < row_bytes || src_row_stride_bytes < row_bytes) return SLORA_ERR_BAD_SHAPE;
+  if (n_bufs == 0 || n_rows == 0 || row_bytes == 0) return SLORA_OK;
+  if (dst_bufs == nullptr || src_bufs == nullptr || loc == nullptr) return SLORA_ERR_NULL_POINTER;
+  for (int i = 0; i < n_bufs; ++i)
+    if (dst_bufs[i] == nullptr || src_bufs[i] == nullptr) return SLORA_ERR_NULL_POINTER;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  for (int b0 = 0; b0 < n_bufs; b0 += kScatterBufs) {
+    ScatterArgs p{};
+    p.n_bufs = n_bufs - b0 < kScatterBufs ? n_bufs - b0 : kScatterBufs;
+    bool vec = (row_bytes % 16 == 0) && (dst_row_stride_bytes % 16 == 0) && (src_row_stride_bytes % 16 == 0);
+    for (int i = 0; i < p.n_bufs; ++i) {
+      p.dst[i] = dst_bufs[b0 + i];
+      p.src[i] = src_bufs[b0 + i];
+      vec = vec && aligned16(p.dst[i]) && aligned16(p.src[i]);
+    }
+    p.loc = loc;
+    p.n_rows = n_rows;
+    p.n_pages = n_pages;
+    p.row_bytes = row_bytes;
+    p.dst_stride = dst_row_stride_bytes;
+    p.src_stride = src_row_stride_bytes;
+    p.vec_ok = vec ? 1 : 0;
+    const int64_t grid = n_rows * p.n_bufs;
+    if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(pool_scatter_kernel, dim3((uint32_t)grid), dim3(256), 0, s, p);
+    if (hipGetLastError() != hipSuccess) return SLORA_ERR_LAUNCH;
+  }
+  return SLORA_OK;
+}
+
+int slora_var_len_copy(const int64_t* old_a_start, const int64_t* old_a_len, const int64_t* old_a_loc,
+                       const int64_t* new_a_start, int64_t* new_a_loc, int64_t n_adapters, int64_t n_old_loc,
+                       int64_t n_new_loc, void* stream) {
+  using namespace slora;
+  if (n_adapters < 0 || n_old_loc < 0 || n_new_loc < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n_adapters == 0) return SLORA_OK;
+  if (old_a_start == nullptr || old_a_len == nullptr || old_a_loc == nullptr || new_a_start == nullptr ||
+      new_a_loc == nullptr)
+    return SLORA_ERR_NULL_POINTER;
+  if (n_adapters > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(var_len_copy_kernel, dim3((uint32_t)n_adapters), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), old_a_start, old_a_len, old_a_loc, new_a_start, new_a_loc,
+                     n_old_loc, n_new_loc);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_tables_compact(const slora_tables* tables, const void* a_scaling, int scales_dtype, const uint8_t* keep,
+                         int64_t* new_a_start, int64_t* new_a_len, int64_t* new_a_loc, void* new_a_scaling,
+                         int64_t* removed_pages, int64_t* counts, int64_t* work, void* stream) {
+  using namespace slora;
+  if (tables == nullptr || counts == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (tables->n_adapters < 0 || tables->n_loc < 0) return SLORA_ERR_BAD_SHAPE;
+  if (scales_dtype != SLORA_DTYPE_F16 && scales_dtype != SLORA_DTYPE_BF16 && scales_dtype != SLORA_DTYPE_F32)
+    return SLORA_ERR_BAD_DTYPE;
+  if (tables->n_adapters > 0 &&
+      (tables->a_start == nullptr || tables->a_len == nullptr || a_scaling == nullptr || keep == nullptr ||
+       new_a_start == nullptr || new_a_len == nullptr || new_a_scaling == nullptr || work == nullptr))
+    return SLORA_ERR_NULL_POINTER;
+  if (tables->n_loc > 0 && (tables->a_loc == nullptr || new_a_loc == nullptr || removed_pages == nullptr))
+    return SLORA_ERR_NULL_POINTER;
+  CompactArgs p{};
+  p.a_start = tables->a_start;
+  p.a_len = tables->a_len;
+  p.a_loc = tables->a_loc;
+  p.a_scaling = a_scaling;
+  p.keep = keep;
+  p.new_start = new_a_start;
+  p.new_len = new_a_len;
+  p.new_loc = new_a_loc;
+  p.new_scaling = new_a_scaling;
+  p.removed = removed_pages;
+  p.counts = counts;
+  p.work = work;
+  p.n_adapters = tables->n_adapters;
+  p.n_loc = tables->n_loc;
+  p.scale_bytes = scales_dtype == SLORA_DTYPE_F32 ? 4 : 2;
+  hipLaunchKernelGGL(tables_compact_kernel, dim3(1), dim3(kCompactThreads), 0, reinterpret_cast<hipStream_t>(stream),
+                     p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+}  // extern "C"

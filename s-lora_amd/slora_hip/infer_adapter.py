@@ -1,0 +1,113 @@
+"""Loading adapters into the unified pool and dropping them again: the device
+side of ``InferAdapter`` (slora/server/router/model_infer/infer_adapter.py).
+
+* ``load_rows_into_pool``    -- ``buffer[loc] = rows`` for many buffers in one launch
+                               (``load_lora_A`` / ``load_lora_B``, :43-88).
+* ``launch_var_len_copy``    -- same arguments as ``launch_var_len_copy_triton`` (:274-280).
+* ``compact_adapter_tables`` -- the table rebuild of ``offload_adapters`` (:186-258).
+
+All three are ctypes calls into libslora_hip.so; there is no fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _cabi
+from ._kernels import _DTYPE_CODE, _check_index, _check_input, _stream, _tables
+
+
+def load_rows_into_pool(buffers, rows, loc) -> None:
+    """``buffers[b][loc] = rows[b]`` for every b, in one launch per 64 buffers.
+
+    ``buffers``: pool tensors ``[n_pages, ...]`` of one shape and dtype (e.g.
+    ``key_buffer[l]`` and ``value_buffer[l]`` of every layer); ``rows``: as many
+    tensors ``[len(loc), ...]`` with the same trailing shape (``w_combined[0]``
+    and ``w_combined[1]`` of every layer); ``loc``: int64 page ids on the device.
+    """
+    buffers, rows = list(buffers), list(rows)
+    if len(buffers) != len(rows):
+        raise RuntimeError(f"{len(buffers)} pool buffers but {len(rows)} row blocks")
+    if not buffers:
+        return
+    _check_input(loc, "loc")
+    _check_index(loc, "loc")
+    n_rows = loc.numel()
+    b0 = buffers[0]
+    row_elems = b0[0].numel() if b0.size(0) else 0
+    for i, (b, r) in enumerate(zip(buffers, rows)):
+        _check_input(b, f"buffers[{i}]")
+        _check_input(r, f"rows[{i}]")
+        if b.dtype != b0.dtype or r.dtype != b0.dtype:
+            raise RuntimeError("pool buffers and rows must share one dtype")
+        if b.shape != b0.shape:
+            raise RuntimeError("pool buffers must share one shape")
+        if r.size(0) != n_rows or r.numel() != n_rows * row_elems:
+            raise RuntimeError(f"rows[{i}] must be [{n_rows}, {tuple(b0.shape[1:])}], got {tuple(r.shape)}")
+    row_bytes = row_elems * b0.element_size()
+    lib = _cabi.load_library()
+    n = len(buffers)
+    dst = (C.c_void_p * n)(*[b.data_ptr() for b in buffers])
+    src = (C.c_void_p * n)(*[r.data_ptr() for r in rows])
+    rc = lib.slora_pool_scatter_rows(dst, src, n, loc.data_ptr(), n_rows, row_bytes, row_bytes, row_bytes, b0.size(0),
+                                     _stream(loc))
+    _cabi.check(rc, "load_rows_into_pool")
+
+
+def launch_var_len_copy(old_a_start, old_a_len, old_location, new_a_start, new_a_location) -> None:
+    """``new_a_location[new_a_start[i] + k] = old_location[old_a_start[i] + k]``
+    for ``k < old_a_len[i]`` (infer_adapter.py:261-280)."""
+    for t, n in ((old_a_start, "old_a_start"), (old_a_len, "old_a_len"), (old_location, "old_location"),
+                 (new_a_start, "new_a_start"), (new_a_location, "new_a_location")):
+        _check_input(t, n)
+        _check_index(t, n)
+    n = old_a_start.numel()
+    if old_a_len.numel() != n or new_a_start.numel() != n:
+        raise RuntimeError("old_a_start, old_a_len and new_a_start must have one entry per adapter")
+    lib = _cabi.load_library()
+    rc = lib.slora_var_len_copy(old_a_start.data_ptr(), old_a_len.data_ptr(), old_location.data_ptr(),
+                                new_a_start.data_ptr(), new_a_location.data_ptr(), n, old_location.numel(),
+                                new_a_location.numel(), _stream(old_location))
+    _cabi.check(rc, "launch_var_len_copy")
+
+
+launch_var_len_copy_triton = launch_var_len_copy  # the name the reference imports
+
+
+def compact_adapter_tables(a_start, a_len, a_loc, a_scaling, keep):
+    """Drop the adapters with ``keep[i] == False``.  Returns ``(new_a_start,
+    new_a_len, new_a_loc, new_a_scaling, removed_pages)``: the tables of the
+    kept adapters in their old order and the page ids to give back to the
+    allocator.  One launch and one 32-byte read-back."""
+    for t, n in ((a_start, "a_start"), (a_len, "a_len"), (a_loc, "a_loc")):
+        _check_input(t, n)
+        _check_index(t, n)
+    _check_input(a_scaling, "a_scaling")
+    _check_input(keep, "keep")
+    n = a_start.numel()
+    if a_len.numel() != n or a_scaling.numel() != n or keep.numel() != n:
+        raise RuntimeError("a_start, a_len, a_scaling and keep must have one entry per adapter")
+    if a_scaling.dtype not in _DTYPE_CODE:
+        raise RuntimeError(f"a_scaling must be float16, bfloat16 or float32, got {a_scaling.dtype}")
+    if keep.dtype not in (torch.bool, torch.uint8):
+        raise RuntimeError(f"keep must be a bool or uint8 tensor, got {keep.dtype}")
+    dev = a_start.device
+    n_loc = a_loc.numel()
+    new_start = torch.empty(n, dtype=torch.int64, device=dev)
+    new_len = torch.empty(n, dtype=torch.int64, device=dev)
+    new_loc = torch.empty(n_loc, dtype=torch.int64, device=dev)
+    new_scaling = torch.empty(n, dtype=a_scaling.dtype, device=dev)
+    removed = torch.empty(n_loc, dtype=torch.int64, device=dev)
+    counts = torch.zeros(4, dtype=torch.int64, device=dev)
+    work = torch.empty(max(n, 1), dtype=torch.int64, device=dev)
+    lib = _cabi.load_library()
+    tables = _tables(a_start, a_len, a_loc)
+    rc = lib.slora_tables_compact(C.byref(tables), a_scaling.data_ptr(), _DTYPE_CODE[a_scaling.dtype],
+                                  keep.view(torch.uint8).data_ptr() if keep.dtype == torch.bool else keep.data_ptr(),
+                                  new_start.data_ptr(), new_len.data_ptr(), new_loc.data_ptr(),
+                                  new_scaling.data_ptr(), removed.data_ptr(), counts.data_ptr(), work.data_ptr(),
+                                  _stream(a_start))
+    _cabi.check(rc, "compact_adapter_tables")
+    n_keep, n_keep_loc, _, n_removed_loc = (int(v) for v in counts.cpu())
+    return new_start[:n_keep], new_len[:n_keep], new_loc[:n_keep_loc], new_scaling[:n_keep], removed[:n_removed_loc]

@@ -305,6 +305,40 @@ def test_var_len_copy():
     assert out.tolist() == list(range(1000, 1032)) + list(range(1096, 1300))
 
 
+def test_offload_tables_explicit_and_invariants():
+    """Hand-written expected tables for a 4-adapter case, then on random cases the
+    properties that fix the result: kept adapters keep order, lengths, scaling and
+    their exact page lists; starts are the running sum; kept + removed pages are
+    the old pages, each exactly once."""
+    a_len = np.array([8, 4, 12, 4], np.int64)
+    a_start = np.array([0, 8, 12, 24], np.int64)
+    a_loc = np.arange(100, 128, dtype=np.int64)[::-1].copy()   # 127 .. 100
+    scal = np.array([2.0, 4.0, 1.0, 8.0], np.float32)
+    ns, nl, nloc, nsc, rem = O.ref_offload_tables(a_start, a_len, a_loc, scal, [True, False, True, False])
+    assert ns.tolist() == [0, 8] and nl.tolist() == [8, 12] and nsc.tolist() == [2.0, 1.0]
+    assert nloc.tolist() == list(range(127, 119, -1)) + list(range(115, 103, -1))
+    assert rem.tolist() == list(range(119, 115, -1)) + list(range(103, 99, -1))
+    # nothing kept / everything kept
+    ns, nl, nloc, nsc, rem = O.ref_offload_tables(a_start, a_len, a_loc, scal, [False] * 4)
+    assert ns.size == nl.size == nloc.size == nsc.size == 0 and rem.tolist() == a_loc.tolist()
+    ns, nl, nloc, nsc, rem = O.ref_offload_tables(a_start, a_len, a_loc, scal, [True] * 4)
+    assert ns.tolist() == a_start.tolist() and nloc.tolist() == a_loc.tolist() and rem.size == 0
+    rng = np.random.default_rng(5)
+    for _ in range(20):
+        n = int(rng.integers(1, 40))
+        ranks = rng.choice([2, 8, 16, 64, 70], size=n)
+        a_start, a_len, a_loc = O.build_tables(ranks, rng.permutation(100000)[: int(4 * ranks.sum())])
+        scal = rng.standard_normal(n).astype(np.float32)
+        keep = rng.random(n) < 0.6
+        ns, nl, nloc, nsc, rem = O.ref_offload_tables(a_start, a_len, a_loc, scal, keep)
+        left = np.nonzero(keep)[0]
+        assert nl.tolist() == a_len[left].tolist() and nsc.tolist() == scal[left].tolist()
+        assert ns.tolist() == (np.cumsum(nl) - nl).tolist()
+        for k, i in enumerate(left):
+            assert nloc[ns[k]: ns[k] + nl[k]].tolist() == a_loc[a_start[i]: a_start[i] + a_len[i]].tolist()
+        assert sorted(np.concatenate([nloc, rem]).tolist()) == sorted(a_loc.tolist())
+
+
 # ---------------------------------------------------------------------------
 # committed fixture (closed form in float64 on the dense matrices) and CPU baseline
 # ---------------------------------------------------------------------------
