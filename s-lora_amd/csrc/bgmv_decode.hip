@@ -65,6 +65,7 @@ constexpr int kPlanHeaderWords = 16;
 // and expand: [SY_TIMEOUT] set if a wavefront ever gave up waiting, then two
 // counters per (token, projection), used at the first token of a run: shrink
 // workgroups of the run that are done, expand wavefronts of the run that are done.
+// They only grow (by at most 8 * rank / 8 per launch) until the plan is rebuilt.
 constexpr int kSyncHeader = 4;
 enum { SY_TIMEOUT = 1 };
 constexpr int kItemWords = 48;
@@ -697,14 +698,21 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint
   // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
   const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
                       (p.page_elems % (8 * r)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
-  // FUSED: two counters per (first token of the run, projection): shrink workgroups
-  // that have stored their rows, and expand wavefronts that are through with them.
+  // FUSED: two counters per (first token of the run, projection), never reset while
+  // the plan lives: cnt[0] counts shrink workgroups of the run that have stored
+  // their rows (`need` per launch), cnt[1] expand wavefronts of the run that are
+  // through (8 per item, with or without work: 8 * need per launch).  Between
+  // launches both are whole multiples; during launch n cnt[1] stays below
+  // (n + 1) * 8 * need as long as this wavefront has not checked out itself, so its
+  // value tells n, and the rows are complete once cnt[0] reaches (n + 1) * need.
   const int listed = r < p.rank_cap ? r : p.rank_cap;
   const int need = (listed + kRB - 1) / kRB;  // the run's items = its shrink workgroups per projection
   int* cnt = FUSED ? p.sync + kSyncHeader + (it.tok[0] * 4 + p.qkvo0 + proj) * 2 : nullptr;
   if (FUSED && has_work) {
+    const int out = __hip_atomic_load(cnt + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int target = (out / (2 * 4 * need) + 1) * need;
     int spins = 0;
-    while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < need) {
+    while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
       if (++spins > p.spin_limit) {  // never expected; leaves a mark instead of waiting for ever
         p.sync[SY_TIMEOUT] = 1;
         break;
@@ -722,19 +730,8 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint
 #pragma unroll 1
     for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T, FUSED>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
   }
-  if (FUSED) {
-    // Every wavefront of every item of the run checks out (8 per item, with or without
-    // work); the last one has seen all the others finish reading and puts both
-    // counters back to zero for the next launch.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    if ((threadIdx.x & 63) == 0) {
-      const int out = __hip_atomic_fetch_add(cnt + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (out == 2 * 4 * need - 1) {
-        __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(cnt + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-  }
+  if (FUSED && (threadIdx.x & 63) == 0)  // check out; nobody waits for the result
+    __hip_atomic_fetch_add(cnt + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------
@@ -1168,10 +1165,10 @@ __global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p)
 // first expand workgroup starts and a waiting expand wavefront cannot starve the
 // producers it waits for.  A shrink workgroup counts itself in on its run's
 // counter after its rows are stored; an expand wavefront polls that counter before
-// it reads them, and checks out on a second counter when it is done; the last
-// wavefront to check out clears both, so the next launch finds them at zero.
-// There is no counter that every workgroup touches: thousands of device-scope
-// atomics on one address cost more than the launch boundary they replace.
+// it reads them, and checks out on a second counter when it is done (see
+// expand_body).  No atomic returns a value anybody waits for, and there is no
+// counter that every workgroup touches: thousands of device-scope atomics on one
+// address cost more than the launch boundary they replace.
 struct LoraArgs {
   ShrinkArgs s;
   ExpandArgs e;
