@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0
 # a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
 # None where not measured.
 TRAFFIC_BYTES = {
-    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80655596,  # 74364140 read + 6291456 written
-    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70295448,     # the q/k/v launch
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80675465,  # 74384009 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70285414,     # the q/k/v launch
 }
 
 
@@ -387,6 +387,34 @@ def main_load(args, torch, device):
     ms = time_region(graphed(step, torch) if use_graph else step, max(5, args.steps), args.warmup, torch)
     ms_torch = time_region(graphed(torch_step, torch) if use_graph else torch_step, max(5, args.steps), args.warmup,
                            torch)
+    # the allocator call that precedes a load: 256 pages out of a 65536-page map (and back)
+    from slora_hip.infer_adapter import PageAllocator
+    pa = PageAllocator(65536, device)
+    pa.alloc(30000)  # a used prefix, as after some uptime
+    state = pa.mem_state.clone()
+    cum = torch.empty(65536, dtype=torch.int32, device=device)
+    idx = torch.arange(65536, dtype=torch.long, device=device)
+
+    def alloc_free():
+        pa.free(pa.alloc(4 * r))
+
+    def torch_alloc_free():  # mem_allocator.py:34-38, 196
+        torch.cumsum(state, dim=0, dtype=torch.int32, out=cum)
+        sel = idx[torch.logical_and(cum <= 4 * r, state == 1)]
+        state[sel] = 0
+        state[sel] = 1
+
+    def host_us(fn, n=200):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    alloc_us, torch_alloc_us = host_us(alloc_free), host_us(torch_alloc_free)
     nbytes = 2 * (4 * r) * H * 2 * 2 * L  # read + write per adapter
     us = ms * 1e3 / n_adapters
     gbs = nbytes / us / 1e3
@@ -402,6 +430,8 @@ def main_load(args, torch, device):
                      "algorithmic_bytes_per_launch": nbytes, "us_per_launch": round(us, 3)},
         "torch_index_put": {"us_per_adapter": round(ms_torch * 1e3 / n_adapters, 3),
                             "launches_per_adapter": 2 * L},
+        "allocator": {"what": "alloc(256) + free on a 65536-page map, wall time per pair incl. Python",
+                      "us": round(alloc_us, 1), "torch_ops_us": round(torch_alloc_us, 1)},
     }
     print(json.dumps(out), flush=True)
 

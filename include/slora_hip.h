@@ -247,6 +247,32 @@ SLORA_API int slora_tables_compact(const slora_tables* tables, const void* a_sca
                          void* new_a_scaling, int64_t* removed_pages, int64_t* counts, int64_t* work,
                          void* stream);
 
+/* ---- page allocator over the pool's free map ---------------------------------
+ * mem_state: one byte per pool page, 1 = free (the reference's torch.bool
+ * `mem_state`, slora/common/mem_allocator.py:222).  `workspace` is device memory of
+ * slora_pool_alloc_workspace_bytes(tot_size) bytes owned by the caller; `result`
+ * is two device int64.  The host keeps the free-page count itself, as the
+ * reference does (`can_use_mem_size`). */
+SLORA_API int64_t slora_pool_alloc_workspace_bytes(int64_t tot_size);
+
+/* MemoryAllocator.alloc (mem_allocator.py:30-39): the first `need` free pages in
+ * index order are written to out_index (ascending) and marked used; result[0] =
+ * pages handed out (fewer than `need` only if the map has fewer free pages). */
+SLORA_API int slora_pool_alloc(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index,
+                     int64_t* result, void* workspace, void* stream);
+
+/* MemoryAllocator.alloc_contiguous (mem_allocator.py:42-59): the first start s with
+ * pages [s, s + need) all free; they are marked used and listed in out_index.
+ * result[0] = s or -1 if there is no such run (nothing is changed then),
+ * result[1] = pages handed out. */
+SLORA_API int slora_pool_alloc_contiguous(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index,
+                                int64_t* result, void* workspace, void* stream);
+
+/* MemoryAllocator.free (mem_allocator.py:185-199): mem_state[free_index] = 1;
+ * ids outside the map are skipped. */
+SLORA_API int slora_pool_free(uint8_t* mem_state, int64_t tot_size, const int64_t* free_index, int64_t n,
+                    void* stream);
+
 #ifdef __cplusplus
 }
 #endif

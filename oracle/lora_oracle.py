@@ -356,6 +356,43 @@ def ref_offload_tables(a_start, a_len, a_loc, a_scaling, keep):
 
 
 # ----------------------------------------------------------------------------
+# page allocator over the free map (slora/common/mem_allocator.py)
+# ----------------------------------------------------------------------------
+def ref_alloc(mem_state, need_size: int):
+    """``MemoryAllocator.alloc`` (mem_allocator.py:30-39) on a 0/1 numpy map
+    (1 = free), in place: ``select = (cumsum(mem_state) <= need_size) &
+    (mem_state == 1)``; the selected pages are marked used and returned."""
+    cum = np.cumsum(mem_state.astype(np.int64))
+    select = np.nonzero((cum <= need_size) & (mem_state == 1))[0].astype(np.int64)
+    mem_state[select] = 0
+    return select
+
+
+def ref_alloc_contiguous(mem_state, need_size: int):
+    """``MemoryAllocator.alloc_contiguous`` (mem_allocator.py:42-59), in place:
+    window sums from the running sum, the first start whose window of
+    ``need_size`` pages is all free; ``None`` if there is none, else
+    ``(select_index, start, end)``."""
+    tot = mem_state.size
+    if need_size > tot:
+        return None
+    cum = np.cumsum(mem_state.astype(np.int64))
+    loc_sums = cum[need_size - 1:tot] - cum[0:tot - need_size + 1] + mem_state[0:tot - need_size + 1]
+    can_use = np.nonzero(loc_sums == need_size)[0]
+    if can_use.size == 0:
+        return None
+    start = int(can_use[0])
+    select = np.arange(start, start + need_size, dtype=np.int64)
+    mem_state[select] = 0
+    return select, start, start + need_size
+
+
+def ref_free(mem_state, free_index):
+    """``MemoryAllocator.free`` (mem_allocator.py:185-199): ``mem_state[free_index] = 1``."""
+    mem_state[np.asarray(free_index, dtype=np.int64)] = 1
+
+
+# ----------------------------------------------------------------------------
 # the reference's torch path on host cores (CPU baseline of the benchmark)
 # ----------------------------------------------------------------------------
 class BmmCpuLayer:

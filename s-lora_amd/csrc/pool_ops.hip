@@ -10,8 +10,12 @@
 //   slora_tables_compact      the index tables after some adapters are dropped, and the
 //                             page ids they give back (infer_adapter.py:186-258)
 //
-// All three are plain byte/integer movement, bound by HBM bandwidth (the first)
-// or by a handful of dependent round trips (the other two).
+//   slora_pool_alloc / slora_pool_alloc_contiguous / slora_pool_free
+//                             the page allocator over the pool's free map
+//                             (slora/common/mem_allocator.py:30-59, 185-199)
+//
+// All of it is plain byte/integer movement, bound by HBM bandwidth (the first) or
+// by a handful of dependent round trips (the rest).
 
 #include "common.hpp"
 #include "cabi_util.hpp"
@@ -193,6 +197,222 @@ __global__ __launch_bounds__(kCompactThreads) void tables_compact_kernel(const C
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// page allocator over the free map (1 byte per page, 1 = free)
+// ---------------------------------------------------------------------------
+constexpr int kMapThreads = 256;
+constexpr int kMapPerThread = 16;                            // one 16-byte load of the map per thread
+constexpr int kMapBlock = kMapThreads * kMapPerThread;       // pages per workgroup
+constexpr int kMapWaves = kMapThreads / kWave;
+
+// the 16 map bytes of this thread (0 beyond the end), as 0/1 flags
+__device__ __forceinline__ void map_load16(const uint8_t* __restrict__ map, int64_t tot, int64_t base, int (&f)[16],
+                                           bool vec) {
+  if (vec && base + 16 <= tot) {
+    const u32x4 v = ldg16(map + base);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] = ((v[i >> 2] >> ((i & 3) * 8)) & 0xffu) != 0 ? 1 : 0;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) f[i] = (base + i < tot && map[base + i] != 0) ? 1 : 0;
+  }
+}
+
+// workgroup b: number of free pages, and (for the contiguous search) the index of its
+// last used page (-1: none), into block_free[b] / block_last_used[b]
+__global__ __launch_bounds__(kMapThreads) void map_block_stats_kernel(const uint8_t* __restrict__ map, int64_t tot,
+                                                                      int* __restrict__ block_free,
+                                                                      int64_t* __restrict__ block_last_used, int vec) {
+  __shared__ int s_cnt[kMapWaves];
+  __shared__ long long s_last[kMapWaves];
+  const int64_t base = (int64_t)blockIdx.x * kMapBlock + (int64_t)threadIdx.x * kMapPerThread;
+  int f[16];
+  map_load16(map, tot, base, f, vec != 0);
+  int cnt = 0;
+  long long last = -1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    cnt += f[i];
+    if (!f[i] && base + i < tot) last = base + i;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    cnt += __shfl_xor(cnt, o, kWave);
+    const long long ol = __shfl_xor(last, o, kWave);
+    last = ol > last ? ol : last;
+  }
+  if ((threadIdx.x & 63) == 0) {
+    s_cnt[threadIdx.x >> 6] = cnt;
+    s_last[threadIdx.x >> 6] = last;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int c = 0;
+    long long l = -1;
+    for (int w = 0; w < kMapWaves; ++w) {
+      c += s_cnt[w];
+      l = s_last[w] > l ? s_last[w] : l;
+    }
+    block_free[blockIdx.x] = c;
+    if (block_last_used != nullptr) block_last_used[blockIdx.x] = l;
+  }
+}
+
+// `mem_cum_sum <= need_size and mem_state == 1` (mem_allocator.py:34-38): the free
+// pages whose rank among the free pages is <= need, in index order, are written to
+// out[rank - 1] and marked used.  result[0] = pages handed out.
+__global__ __launch_bounds__(kMapThreads) void map_alloc_kernel(uint8_t* __restrict__ map, int64_t tot, int64_t need,
+                                                                const int* __restrict__ block_free, int n_blocks,
+                                                                int64_t* __restrict__ out, int64_t* __restrict__ result,
+                                                                int vec) {
+  __shared__ long long s_part[kMapWaves];
+  __shared__ int s_scan[kMapWaves];
+  // free pages in front of this workgroup, and in total
+  long long before = 0, total = 0;
+  for (int b = threadIdx.x; b < n_blocks; b += kMapThreads) {
+    const int c = block_free[b];
+    if (b < (int)blockIdx.x) before += c;
+    total += c;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    before += __shfl_xor(before, o, kWave);
+    total += __shfl_xor(total, o, kWave);
+  }
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = before;
+  __syncthreads();
+  before = 0;
+  for (int w = 0; w < kMapWaves; ++w) before += s_part[w];
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = total;
+  __syncthreads();
+  total = 0;
+  for (int w = 0; w < kMapWaves; ++w) total += s_part[w];
+  if (blockIdx.x == 0 && threadIdx.x == 0) result[0] = total < need ? total : need;
+  if (before >= need) return;  // uniform
+
+  const int64_t base = (int64_t)blockIdx.x * kMapBlock + (int64_t)threadIdx.x * kMapPerThread;
+  int f[16];
+  map_load16(map, tot, base, f, vec != 0);
+  int mine = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) mine += f[i];
+  // exclusive scan of `mine` over the workgroup
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc = mine;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  if (lane == kWave - 1) s_scan[wave] = inc;
+  __syncthreads();
+  long long rank = before + inc - mine;  // free pages in front of this thread's first page
+  for (int w = 0; w < wave; ++w) rank += s_scan[w];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    if (f[i]) {
+      ++rank;
+      if (rank <= need) {
+        out[rank - 1] = base + i;
+        map[base + i] = 0;
+      }
+    }
+  }
+}
+
+// First start s with pages [s, s + need) all free (mem_allocator.py:45-52).  A page i
+// ends such a window iff the nearest used page at or before i lies before i - need + 1.
+// Every workgroup takes the last used page in front of it from block_last_used, scans
+// its own pages and proposes the smallest start it sees with a 64-bit atomic min.
+__global__ __launch_bounds__(kMapThreads) void map_find_run_kernel(const uint8_t* __restrict__ map, int64_t tot,
+                                                                   int64_t need,
+                                                                   const int64_t* __restrict__ block_last_used,
+                                                                   unsigned long long* __restrict__ best, int vec) {
+  __shared__ long long s_last[kMapWaves];
+  long long prev = -1;  // last used page in front of this workgroup
+  for (int b = threadIdx.x; b < (int)blockIdx.x; b += kMapThreads) {
+    const long long l = block_last_used[b];
+    prev = l > prev ? l : prev;
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const long long ol = __shfl_xor(prev, o, kWave);
+    prev = ol > prev ? ol : prev;
+  }
+  if ((threadIdx.x & 63) == 0) s_last[threadIdx.x >> 6] = prev;
+  __syncthreads();
+  prev = -1;
+  for (int w = 0; w < kMapWaves; ++w) prev = s_last[w] > prev ? s_last[w] : prev;
+  __syncthreads();
+
+  const int64_t base = (int64_t)blockIdx.x * kMapBlock + (int64_t)threadIdx.x * kMapPerThread;
+  int f[16];
+  map_load16(map, tot, base, f, vec != 0);
+  long long mine = -1;  // last used page among this thread's pages
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    if (!f[i] && base + i < tot) mine = base + i;
+  // inclusive max-scan over the workgroup, then shifted to "in front of this thread"
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  long long run = mine;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const long long up = __shfl_up(run, o, kWave);
+    if (lane >= o) run = up > run ? up : run;
+  }
+  if (lane == kWave - 1) s_last[wave] = run;
+  __syncthreads();
+  long long front = __shfl_up(run, 1, kWave);
+  if (lane == 0) front = -1;
+  front = front > prev ? front : prev;
+  for (int w = 0; w < wave; ++w) front = s_last[w] > front ? s_last[w] : front;
+  long long last_used = front;
+  unsigned long long cand = ~0ull;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const long long idx = base + i;
+    if (idx < tot) {
+      if (!f[i]) last_used = idx;
+      const long long start = idx - need + 1;
+      if (f[i] && start >= 0 && last_used < start && (unsigned long long)start < cand) cand = (unsigned long long)start;
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) {
+    const unsigned long long oc = __shfl_xor(cand, o, kWave);
+    cand = oc < cand ? oc : cand;
+  }
+  if (lane == 0 && cand != ~0ull) atomicMin(best, cand);
+}
+
+// pages [*best, *best + need) are marked used and listed; result = {start or -1, pages}
+__global__ __launch_bounds__(kMapThreads) void map_take_run_kernel(uint8_t* __restrict__ map, int64_t tot, int64_t need,
+                                                                   const unsigned long long* __restrict__ best,
+                                                                   int64_t* __restrict__ out,
+                                                                   int64_t* __restrict__ result) {
+  const unsigned long long b = *best;
+  const bool found = b != ~0ull && (long long)b + need <= tot;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    result[0] = found ? (int64_t)b : -1;
+    result[1] = found ? need : 0;
+  }
+  if (!found) return;
+  for (int64_t k = (int64_t)blockIdx.x * kMapThreads + threadIdx.x; k < need; k += (int64_t)gridDim.x * kMapThreads) {
+    out[k] = (int64_t)b + k;
+    map[(int64_t)b + k] = 0;
+  }
+}
+
+__global__ __launch_bounds__(256) void map_init_best_kernel(unsigned long long* best) { *best = ~0ull; }
+
+// mem_state[free_index] = 1 (mem_allocator.py:185-199); ids outside the map are skipped
+__global__ __launch_bounds__(256) void map_free_kernel(uint8_t* __restrict__ map, int64_t tot,
+                                                       const int64_t* __restrict__ idx, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) {
+    const int64_t pg = idx[i];
+    if ((uint64_t)pg < (uint64_t)tot) map[pg] = 1;
+  }
+}
+
 }  // namespace
 }  // namespace slora
 
@@ -281,6 +501,75 @@ int slora_tables_compact(const slora_tables* tables, const void* a_scaling, int 
   p.scale_bytes = scales_dtype == SLORA_DTYPE_F32 ? 4 : 2;
   hipLaunchKernelGGL(tables_compact_kernel, dim3(1), dim3(kCompactThreads), 0, reinterpret_cast<hipStream_t>(stream),
                      p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int64_t slora_pool_alloc_workspace_bytes(int64_t tot_size) {
+  if (tot_size < 0) return SLORA_ERR_BAD_SHAPE;
+  const int64_t nb = (tot_size + slora::kMapBlock - 1) / slora::kMapBlock;
+  return 16 + nb * 4 + 8 + nb * 8;  // best start, free counts, (alignment), last used pages
+}
+
+int slora_pool_alloc(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index, int64_t* result,
+                     void* workspace, void* stream) {
+  using namespace slora;
+  if (tot_size < 0 || need < 0) return SLORA_ERR_BAD_SHAPE;
+  if (result == nullptr || workspace == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (tot_size > 0 && mem_state == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (need > 0 && out_index == nullptr) return SLORA_ERR_NULL_POINTER;
+  const int64_t nb = (tot_size + kMapBlock - 1) / kMapBlock;
+  if (nb > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  int* block_free = reinterpret_cast<int*>(static_cast<char*>(workspace) + 16);
+  const int vec = aligned16(mem_state) ? 1 : 0;
+  if (nb == 0) {
+    hipLaunchKernelGGL(map_alloc_kernel, dim3(1), dim3(kMapThreads), 0, s, mem_state, tot_size, need, block_free, 0,
+                       out_index, result, vec);
+    return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL(map_block_stats_kernel, dim3((uint32_t)nb), dim3(kMapThreads), 0, s, mem_state, tot_size,
+                     block_free, static_cast<int64_t*>(nullptr), vec);
+  hipLaunchKernelGGL(map_alloc_kernel, dim3((uint32_t)nb), dim3(kMapThreads), 0, s, mem_state, tot_size, need,
+                     block_free, (int)nb, out_index, result, vec);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_alloc_contiguous(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index,
+                                int64_t* result, void* workspace, void* stream) {
+  using namespace slora;
+  if (tot_size < 0 || need <= 0) return SLORA_ERR_BAD_SHAPE;
+  if (result == nullptr || workspace == nullptr || out_index == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (tot_size > 0 && mem_state == nullptr) return SLORA_ERR_NULL_POINTER;
+  const int64_t nb = (tot_size + kMapBlock - 1) / kMapBlock;
+  if (nb > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  unsigned long long* best = static_cast<unsigned long long*>(workspace);
+  int* block_free = reinterpret_cast<int*>(static_cast<char*>(workspace) + 16);
+  int64_t* block_last = reinterpret_cast<int64_t*>(static_cast<char*>(workspace) + 16 + ((nb * 4 + 7) / 8) * 8);
+  const int vec = aligned16(mem_state) ? 1 : 0;
+  hipLaunchKernelGGL(map_init_best_kernel, dim3(1), dim3(1), 0, s, best);
+  if (nb > 0) {
+    hipLaunchKernelGGL(map_block_stats_kernel, dim3((uint32_t)nb), dim3(kMapThreads), 0, s, mem_state, tot_size,
+                       block_free, block_last, vec);
+    hipLaunchKernelGGL(map_find_run_kernel, dim3((uint32_t)nb), dim3(kMapThreads), 0, s, mem_state, tot_size, need,
+                       block_last, best, vec);
+  }
+  int64_t grid = (need + kMapThreads - 1) / kMapThreads;
+  if (grid > 1024) grid = 1024;
+  hipLaunchKernelGGL(map_take_run_kernel, dim3((uint32_t)grid), dim3(kMapThreads), 0, s, mem_state, tot_size, need,
+                     best, out_index, result);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_free(uint8_t* mem_state, int64_t tot_size, const int64_t* free_index, int64_t n, void* stream) {
+  using namespace slora;
+  if (tot_size < 0 || n < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n == 0) return SLORA_OK;
+  if (mem_state == nullptr || free_index == nullptr) return SLORA_ERR_NULL_POINTER;
+  const int64_t grid = (n + 255) / 256;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(map_free_kernel, dim3((uint32_t)grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     mem_state, tot_size, free_index, n);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 

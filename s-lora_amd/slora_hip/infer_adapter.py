@@ -6,7 +6,10 @@ side of ``InferAdapter`` (slora/server/router/model_infer/infer_adapter.py).
 * ``launch_var_len_copy``    -- same arguments as ``launch_var_len_copy_triton`` (:274-280).
 * ``compact_adapter_tables`` -- the table rebuild of ``offload_adapters`` (:186-258).
 
-All three are ctypes calls into libslora_hip.so; there is no fallback.
+* ``PageAllocator``          -- ``MemoryAllocator.alloc / alloc_contiguous / free``
+                               (slora/common/mem_allocator.py:30-59, 185-199) on the device.
+
+All of them are ctypes calls into libslora_hip.so; there is no fallback.
 """
 from __future__ import annotations
 
@@ -111,3 +114,66 @@ def compact_adapter_tables(a_start, a_len, a_loc, a_scaling, keep):
     _cabi.check(rc, "compact_adapter_tables")
     n_keep, n_keep_loc, _, n_removed_loc = (int(v) for v in counts.cpu())
     return new_start[:n_keep], new_len[:n_keep], new_loc[:n_keep_loc], new_scaling[:n_keep], removed[:n_removed_loc]
+
+
+class PageAllocator:
+    """The free map of the unified pool and the three operations the serving loop
+    uses on it (``MemoryAllocator`` of slora/common/mem_allocator.py without the
+    buffers): ``mem_state`` is a bool tensor, True = free, exactly the reference's;
+    ``can_use_mem_size`` is kept on the host as the reference keeps it."""
+
+    def __init__(self, tot_size: int, device="cuda"):
+        self.tot_size = int(tot_size)
+        self.device = torch.device(device)
+        self.mem_state = torch.ones((self.tot_size,), dtype=torch.bool, device=self.device)
+        self.can_use_mem_size = self.tot_size
+        lib = _cabi.load_library()
+        nbytes = int(lib.slora_pool_alloc_workspace_bytes(self.tot_size))
+        self._work = torch.empty((nbytes + 7) // 8, dtype=torch.int64, device=self.device)
+        self._result = torch.zeros(2, dtype=torch.int64, device=self.device)
+
+    def _state_ptr(self) -> int:
+        return self.mem_state.data_ptr()
+
+    def alloc(self, need_size: int) -> torch.Tensor:
+        need_size = int(need_size)
+        if need_size > self.can_use_mem_size:
+            raise Exception(f'warn no enough pool space: need_size {need_size} left_size {self.can_use_mem_size}')
+        out = torch.empty(need_size, dtype=torch.int64, device=self.device)
+        lib = _cabi.load_library()
+        rc = lib.slora_pool_alloc(self._state_ptr(), self.tot_size, need_size, out.data_ptr(),
+                                  self._result.data_ptr(), self._work.data_ptr(), _stream(self.mem_state))
+        _cabi.check(rc, "PageAllocator.alloc")
+        self.can_use_mem_size -= need_size
+        return out
+
+    def alloc_contiguous(self, need_size: int):
+        need_size = int(need_size)
+        if need_size > self.can_use_mem_size:
+            raise Exception(f'warn no enough pool space: need_size {need_size} left_size {self.can_use_mem_size}')
+        if need_size <= 0:
+            raise RuntimeError("need_size must be positive")
+        out = torch.empty(need_size, dtype=torch.int64, device=self.device)
+        lib = _cabi.load_library()
+        rc = lib.slora_pool_alloc_contiguous(self._state_ptr(), self.tot_size, need_size, out.data_ptr(),
+                                             self._result.data_ptr(), self._work.data_ptr(),
+                                             _stream(self.mem_state))
+        _cabi.check(rc, "PageAllocator.alloc_contiguous")
+        start = int(self._result[0].item())  # the reference reads the start back as well (mem_allocator.py:57)
+        if start < 0:
+            return None
+        self.can_use_mem_size -= need_size
+        return out, start, start + need_size
+
+    def free(self, free_index: torch.Tensor) -> None:
+        _check_input(free_index, "free_index")
+        _check_index(free_index, "free_index")
+        lib = _cabi.load_library()
+        rc = lib.slora_pool_free(self._state_ptr(), self.tot_size, free_index.data_ptr(), free_index.numel(),
+                                 _stream(self.mem_state))
+        _cabi.check(rc, "PageAllocator.free")
+        self.can_use_mem_size += free_index.shape[0]
+
+    def free_all(self) -> None:
+        self.mem_state[:] = True
+        self.can_use_mem_size = self.tot_size

@@ -339,6 +339,37 @@ def test_offload_tables_explicit_and_invariants():
         assert sorted(np.concatenate([nloc, rem]).tolist()) == sorted(a_loc.tolist())
 
 
+def test_allocator_against_brute_force():
+    """ref_alloc / ref_alloc_contiguous / ref_free against the plain definitions:
+    the first n free pages in index order; the smallest s with pages s..s+n-1 all
+    free (tried one start at a time)."""
+    rng = np.random.default_rng(9)
+    for _ in range(200):
+        tot = int(rng.integers(1, 60))
+        state = (rng.random(tot) < rng.random()).astype(np.uint8)
+        need = int(rng.integers(0, tot + 2))
+        free = [i for i in range(tot) if state[i]]
+        s1 = state.copy()
+        got = O.ref_alloc(s1, need)
+        assert got.tolist() == free[:need]
+        exp = state.copy()
+        exp[free[:need]] = 0
+        assert np.array_equal(s1, exp)
+        if need >= 1:
+            s2 = state.copy()
+            res = O.ref_alloc_contiguous(s2, need)
+            starts = [s for s in range(0, tot - need + 1) if all(state[s + k] for k in range(need))]
+            if not starts:
+                assert res is None and np.array_equal(s2, state)
+            else:
+                sel, a, b = res
+                assert (a, b) == (starts[0], starts[0] + need) and sel.tolist() == list(range(a, b))
+                assert s2[a:b].sum() == 0 and np.array_equal(np.delete(s2, np.arange(a, b)), np.delete(state, np.arange(a, b)))
+        s3 = s1.copy()
+        O.ref_free(s3, got)
+        assert np.array_equal(s3, state)
+
+
 # ---------------------------------------------------------------------------
 # committed fixture (closed form in float64 on the dense matrices) and CPU baseline
 # ---------------------------------------------------------------------------

@@ -102,6 +102,51 @@ def test_var_len_copy_and_table_compaction(gpu, n, ranks):
             assert np.array_equal(out.cpu().numpy(), nloc)
 
 
+@pytest.mark.parametrize("tot", [1, 37, 4096, 4097, 70000, 262144])
+def test_page_allocator_equals_the_reference_allocator(gpu, tot):
+    """alloc / alloc_contiguous / free on the device against the oracle's restatement
+    of MemoryAllocator, bit for bit, over a random sequence of calls on maps that
+    cross the kernels' 4096-page blocks."""
+    from slora_hip.infer_adapter import PageAllocator
+    rng = np.random.default_rng(tot)
+    pa = PageAllocator(tot, gpu)
+    state = np.ones(tot, np.uint8)
+    held = []
+    for step in range(40):
+        free_now = int(state.sum())
+        op = rng.integers(0, 4)
+        if op == 0 and free_now:
+            need = int(rng.integers(0, min(free_now, max(1, tot // 3)) + 1))
+            exp = O.ref_alloc(state, need)
+            got = pa.alloc(need)
+            assert np.array_equal(got.cpu().numpy(), exp), (step, "alloc", need)
+            held.append(exp)
+        elif op == 1 and free_now:
+            need = int(rng.integers(1, min(free_now, max(1, tot // 8)) + 1))
+            exp = O.ref_alloc_contiguous(state, need)
+            got = pa.alloc_contiguous(need)
+            if exp is None:
+                assert got is None, (step, "contiguous", need)
+            else:
+                assert got is not None and (got[1], got[2]) == (exp[1], exp[2]), (step, "contiguous", need)
+                assert np.array_equal(got[0].cpu().numpy(), exp[0])
+                held.append(exp[0])
+        elif held:
+            # give back a random half of one earlier allocation, scattered
+            blk = held.pop(int(rng.integers(0, len(held))))
+            if blk.size:
+                pick = rng.permutation(blk)[: max(1, blk.size // 2)]
+                rest = np.setdiff1d(blk, pick)
+                O.ref_free(state, pick)
+                pa.free(torch.from_numpy(pick).to(gpu))
+                if rest.size:
+                    held.append(rest)
+        assert np.array_equal(pa.mem_state.cpu().numpy().astype(np.uint8), state), step
+        assert pa.can_use_mem_size == int(state.sum())
+    with pytest.raises(Exception, match="no enough pool space"):
+        pa.alloc(pa.can_use_mem_size + 1)
+
+
 def test_pool_ops_reject_bad_arguments(gpu):
     from slora_hip.infer_adapter import compact_adapter_tables, launch_var_len_copy, load_rows_into_pool
     buf = torch.zeros((10, 2, 8), dtype=torch.float16, device=gpu)
