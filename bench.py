@@ -415,6 +415,23 @@ def main_load(args, torch, device):
         return (time.perf_counter() - t0) / n * 1e6
 
     alloc_us, torch_alloc_us = host_us(alloc_free), host_us(torch_alloc_free)
+
+    # merging one rank-64 adapter into the four [H, H] base matrices of a layer and taking it out again
+    from slora_hip.infer_adapter import merge_adapter, unmerge_adapter
+    a_start = torch.zeros(1, dtype=torch.int64, device=device)
+    a_len = torch.full((1,), 4 * r, dtype=torch.int64, device=device)
+    a_scal = torch.full((1,), 0.25, dtype=torch.float16, device=device)
+    n_w = 4
+    weights = [[torch.randn((H, H), device=device, dtype=torch.float32).to(torch.float16) for _ in range(4)]
+               for _ in range(n_w)]
+
+    def merge_unmerge():
+        for l in range(n_w):
+            merge_adapter(weights[l], bufs[l], bufs[L + l], a_start, a_len, locs[0], a_scal, 0)
+            unmerge_adapter(weights[l], bufs[l], bufs[L + l], a_start, a_len, locs[0], a_scal, 0)
+
+    merge_ms = time_region(merge_unmerge, 5, 2, torch) / (2 * n_w)
+    merge_bytes = 4 * (2 * H * H * 2 + 2 * r * H * 2)
     nbytes = 2 * (4 * r) * H * 2 * 2 * L  # read + write per adapter
     us = ms * 1e3 / n_adapters
     gbs = nbytes / us / 1e3
@@ -430,6 +447,10 @@ def main_load(args, torch, device):
                      "algorithmic_bytes_per_launch": nbytes, "us_per_launch": round(us, 3)},
         "torch_index_put": {"us_per_adapter": round(ms_torch * 1e3 / n_adapters, 3),
                             "launches_per_adapter": 2 * L},
+        "merge_adapter": {"what": "rank-64 adapter into q, k, v, o [4096, 4096] of one layer (4 gathers + 4 launches)",
+                          "us_per_layer": round(merge_ms * 1e3, 1), "bytes_per_layer": merge_bytes,
+                          "GBps": round(merge_bytes / merge_ms / 1e6, 1),
+                          "frac": round(merge_bytes / merge_ms / 1e6 / HBM_PEAK_GBS, 4)},
         "allocator": {"what": "alloc(256) + free on a 65536-page map, wall time per pair incl. Python",
                       "us": round(alloc_us, 1), "torch_ops_us": round(torch_alloc_us, 1)},
     }

@@ -247,6 +247,17 @@ SLORA_API int slora_tables_compact(const slora_tables* tables, const void* a_sca
                          void* new_a_scaling, int64_t* removed_pages, int64_t* counts, int64_t* work,
                          void* stream);
 
+/* A_p of one adapter as a dense row-major (h, out_cols) matrix of 16-bit elements:
+ * out[k, d] = pool[a_loc[first + d]][k] for d < rank, 0 for rank <= d < out_cols.
+ * `first` = a_start[adapter] + qkvo * rank.  This is the unpacking of
+ * slora/models/peft/lora_single_batch_infer.py:38-46
+ * (`key_buffer[l][loc[p r:(p+1) r]].reshape(r, H).transpose(0, 1)`), the left
+ * operand when an adapter is merged into the base weights (:60-93): with it,
+ * W_p += scaling * A_p B_p is slora_sgmm_expand with x = A_p, o = W_p, one request
+ * covering all h rows, and unmerging is the same call with the scale negated. */
+SLORA_API int slora_pool_gather_a(void* out, int64_t out_cols, const void* pool, const int64_t* a_loc, int64_t n_loc,
+                        int64_t first, int64_t rank, int64_t h, int64_t page_elems, int64_t n_pages, void* stream);
+
 /* ---- page allocator over the pool's free map ---------------------------------
  * mem_state: one byte per pool page, 1 = free (the reference's torch.bool
  * `mem_state`, slora/common/mem_allocator.py:222).  `workspace` is device memory of

@@ -355,6 +355,17 @@ def ref_offload_tables(a_start, a_len, a_loc, a_scaling, keep):
     return new_start, new_len, new_loc, np.asarray(a_scaling)[left], removed
 
 
+def ref_merge_adapter(W, A, B, scaling: float, sign: float = 1.0, dtype: str = "f16"):
+    """``LoraPEFTBatchInfer.merge_adapter`` / ``unmerge_adapter`` for one projection
+    (lora_single_batch_infer.py:60-93) with the reference's rounding points:
+    ``b = T(B * scaling)`` (:68), ``ab = T(A @ b)`` (float accumulate inside bmm,
+    :69), ``W = T(W +- ab)`` (:72-75).  ``W``: (H, H_out), ``A``: (H, r), ``B``:
+    (r, H_out); returns the new W as float32 holding storage-type values."""
+    b = round_to(np.asarray(B, np.float32) * np.float32(scaling), dtype)
+    ab = round_to((np.asarray(A, np.float64) @ b.astype(np.float64)).astype(np.float32), dtype)
+    return round_to(np.asarray(W, np.float32) + np.float32(sign) * ab, dtype)
+
+
 # ----------------------------------------------------------------------------
 # page allocator over the free map (slora/common/mem_allocator.py)
 # ----------------------------------------------------------------------------

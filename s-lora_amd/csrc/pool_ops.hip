@@ -10,6 +10,9 @@
 //   slora_tables_compact      the index tables after some adapters are dropped, and the
 //                             page ids they give back (infer_adapter.py:186-258)
 //
+//   slora_pool_gather_a       A_p as a dense (hidden, rank) matrix out of its r pool pages
+//                             (slora/models/peft/lora_single_batch_infer.py:38-46), the
+//                             left operand of merging an adapter into the base weights
 //   slora_pool_alloc / slora_pool_alloc_contiguous / slora_pool_free
 //                             the page allocator over the pool's free map
 //                             (slora/common/mem_allocator.py:30-59, 185-199)
@@ -197,6 +200,34 @@ __global__ __launch_bounds__(kCompactThreads) void tables_compact_kernel(const C
   }
 }
 
+
+// ---------------------------------------------------------------------------
+// A_p out of the pool: out[k, d] = pool[loc[first + d]][k]
+// ---------------------------------------------------------------------------
+// 64 x 64 tiles through LDS: pages are read along k (contiguous), the dense
+// matrix is written along d (contiguous).  Columns r .. out_cols are zero.
+__global__ __launch_bounds__(256) void gather_a_kernel(const uint16_t* __restrict__ pool, int64_t page_elems,
+                                                       int64_t n_pages, const int64_t* __restrict__ loc,
+                                                       int64_t n_loc, int64_t first, int r, int h,
+                                                       uint16_t* __restrict__ out, int out_cols) {
+  __shared__ uint16_t s_t[64][66];
+  const int k0 = blockIdx.x * 64, d0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  for (int dd = ty; dd < 64; dd += 4) {
+    const int d = d0 + dd, k = k0 + tx;
+    uint16_t v = 0;
+    if (d < r && k < h && (uint64_t)(first + d) < (uint64_t)n_loc) {
+      const int64_t page = loc[first + d];
+      if ((uint64_t)page < (uint64_t)n_pages) v = pool[page * page_elems + k];
+    }
+    s_t[dd][tx] = v;
+  }
+  __syncthreads();
+  for (int kk = ty; kk < 64; kk += 4) {
+    const int k = k0 + kk, d = d0 + tx;
+    if (k < h && d < out_cols) out[(int64_t)k * out_cols + d] = s_t[tx][kk];
+  }
+}
 
 // ---------------------------------------------------------------------------
 // page allocator over the free map (1 byte per page, 1 = free)
@@ -501,6 +532,21 @@ int slora_tables_compact(const slora_tables* tables, const void* a_scaling, int 
   p.scale_bytes = scales_dtype == SLORA_DTYPE_F32 ? 4 : 2;
   hipLaunchKernelGGL(tables_compact_kernel, dim3(1), dim3(kCompactThreads), 0, reinterpret_cast<hipStream_t>(stream),
                      p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_gather_a(void* out, int64_t out_cols, const void* pool, const int64_t* a_loc, int64_t n_loc,
+                        int64_t first, int64_t rank, int64_t h, int64_t page_elems, int64_t n_pages, void* stream) {
+  using namespace slora;
+  if (out == nullptr || pool == nullptr || a_loc == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (h < 0 || rank < 0 || out_cols < rank || page_elems < h || n_pages < 0 || first < 0 || n_loc < 0)
+    return SLORA_ERR_BAD_SHAPE;
+  if (h == 0 || out_cols == 0) return SLORA_OK;
+  if (h > (1 << 21) || out_cols > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
+  const dim3 grid((uint32_t)((h + 63) / 64), (uint32_t)((out_cols + 63) / 64));
+  hipLaunchKernelGGL(gather_a_kernel, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(pool), page_elems, n_pages, a_loc, n_loc, first, (int)rank, (int)h,
+                     static_cast<uint16_t*>(out), (int)out_cols);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 

@@ -52,6 +52,7 @@ SIGNATURES = {
     "slora_pool_scatter_rows": (_I, [_P, _P, _I, _P, _I64, _I64, _I64, _I64, _I64, _P]),
     "slora_var_len_copy": (_I, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _P]),
     "slora_tables_compact": (_I, [_TP, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "slora_pool_gather_a": (_I, [_P, _I64, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _P]),
     "slora_pool_alloc_workspace_bytes": (_I64, [_I64]),
     "slora_pool_alloc": (_I, [_P, _I64, _I64, _P, _P, _P, _P]),
     "slora_pool_alloc_contiguous": (_I, [_P, _I64, _I64, _P, _P, _P, _P]),

@@ -9,6 +9,10 @@ side of ``InferAdapter`` (slora/server/router/model_infer/infer_adapter.py).
 * ``PageAllocator``          -- ``MemoryAllocator.alloc / alloc_contiguous / free``
                                (slora/common/mem_allocator.py:30-59, 185-199) on the device.
 
+* ``merge_adapter`` / ``unmerge_adapter`` -- ``W_p +-= scaling * A_p B_p`` for the four
+                               projections of a layer, reading A and B from the pool
+                               (slora/models/peft/lora_single_batch_infer.py:60-93).
+
 All of them are ctypes calls into libslora_hip.so; there is no fallback.
 """
 from __future__ import annotations
@@ -177,3 +181,64 @@ class PageAllocator:
     def free_all(self) -> None:
         self.mem_state[:] = True
         self.can_use_mem_size = self.tot_size
+
+
+def gather_lora_a(key_buffer, a_loc, first: int, rank: int, hidden: int, out_cols: int = 0) -> torch.Tensor:
+    """``A_p`` as a dense ``[hidden, out_cols]`` tensor out of the pool pages
+    ``a_loc[first : first + rank]`` (lora_single_batch_infer.py:38-46); columns
+    ``rank..out_cols`` are zero."""
+    _check_input(key_buffer, "key_buffer")
+    _check_input(a_loc, "a_loc")
+    _check_index(a_loc, "a_loc")
+    if key_buffer.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("key_buffer must be float16 or bfloat16")
+    out_cols = int(out_cols) or int(rank)
+    page_elems = key_buffer[0].numel() if key_buffer.size(0) else 0
+    out = torch.empty((hidden, out_cols), dtype=key_buffer.dtype, device=key_buffer.device)
+    lib = _cabi.load_library()
+    rc = lib.slora_pool_gather_a(out.data_ptr(), out_cols, key_buffer.data_ptr(), a_loc.data_ptr(), a_loc.numel(),
+                                 int(first), int(rank), int(hidden), page_elems, key_buffer.size(0),
+                                 _stream(key_buffer))
+    _cabi.check(rc, "gather_lora_a")
+    return out
+
+
+def merge_adapter(weights, key_buffer, value_buffer, a_start, a_len, a_loc, a_scaling, adapter_idx: int,
+                  sign: float = 1.0) -> None:
+    """One layer of ``LoraPEFTBatchInfer.merge_adapter`` (lora_single_batch_infer.py:60-76):
+    ``weights[p] += sign * scaling * A_p @ B_p`` in place for p in q, k, v, o, with
+    ``weights[p]`` the ``[hidden, h_out_p]`` matrix the base model multiplies
+    activations with, and A, B read from the adapter's pool pages.
+
+    A_p is unpacked by ``gather_lora_a``; the product and the update are the
+    prefill expand kernel with the ``hidden`` rows of A_p standing for tokens of
+    one request (float accumulate, scale applied to the sum, one rounding when
+    the sum is added to W -- the reference rounds ``B * scaling`` and ``A @ B`` to
+    the storage type on the way)."""
+    from .lora_prefill import lora_get_qkvo_fwd_expand
+    if len(weights) != 4:
+        raise RuntimeError("weights must be the q, k, v, o matrices of one layer")
+    start = int(a_start[adapter_idx].item())   # the reference reads these back too (:30-32)
+    rank = int(a_len[adapter_idx].item()) // 4
+    if rank == 0:
+        return
+    dev = key_buffer.device
+    hidden = weights[0].size(0)
+    cols = (rank + 7) // 8 * 8
+    scale = a_scaling if sign == 1.0 else a_scaling * sign
+    seg_start = torch.zeros(1, dtype=torch.int32, device=dev)
+    seg_len = torch.full((1,), hidden, dtype=torch.int32, device=dev)
+    seg_idx = torch.full((1,), int(adapter_idx), dtype=torch.int64, device=dev)
+    page = value_buffer[0].numel()
+    for p in range(4):
+        w_p = weights[p]
+        if w_p.size(0) != hidden or w_p.dtype != key_buffer.dtype:
+            raise RuntimeError(f"weights[{p}] must be [{hidden}, h_out] {key_buffer.dtype}")
+        a_p = gather_lora_a(key_buffer, a_loc, start + p * rank, rank, hidden, cols)
+        lora_get_qkvo_fwd_expand(a_p, value_buffer.view(-1, page), w_p, scale, a_loc, a_start, a_len, seg_start,
+                                 seg_len, seg_idx, w_p.size(1), p, cols, hidden)
+
+
+def unmerge_adapter(weights, key_buffer, value_buffer, a_start, a_len, a_loc, a_scaling, adapter_idx: int) -> None:
+    """``weights[p] -= scaling * A_p @ B_p`` (lora_single_batch_infer.py:78-93)."""
+    merge_adapter(weights, key_buffer, value_buffer, a_start, a_len, a_loc, a_scaling, adapter_idx, sign=-1.0)

@@ -339,6 +339,27 @@ def test_offload_tables_explicit_and_invariants():
         assert sorted(np.concatenate([nloc, rem]).tolist()) == sorted(a_loc.tolist())
 
 
+def test_merge_adapter_closed_form_and_round_trip():
+    """ref_merge_adapter against the dense closed form in float64 (one rounding
+    chain apart), exactly on integer-valued cases, and merge followed by unmerge
+    gives W back exactly where every intermediate is exactly representable."""
+    rng = np.random.default_rng(4)
+    H, Ho, r = 48, 40, 8
+    W = O.round_to(rng.standard_normal((H, Ho)).astype(np.float32), "f16")
+    A = O.round_to(rng.standard_normal((H, r)).astype(np.float32) / 8, "f16")
+    B = O.round_to(rng.standard_normal((r, Ho)).astype(np.float32) / 4, "f16")
+    got = O.ref_merge_adapter(W, A, B, 2.0, 1.0, "f16")
+    exact = W.astype(np.float64) + 2.0 * A.astype(np.float64) @ B.astype(np.float64)
+    np.testing.assert_allclose(got, exact, rtol=2e-3, atol=2e-3)
+    Wi = rng.integers(-8, 9, size=(H, Ho)).astype(np.float32)
+    Ai = rng.integers(-2, 3, size=(H, r)).astype(np.float32)
+    Bi = rng.integers(-2, 3, size=(r, Ho)).astype(np.float32)
+    m = O.ref_merge_adapter(Wi, Ai, Bi, 2.0, 1.0, "f16")
+    assert np.array_equal(m, Wi + 2.0 * Ai @ Bi)
+    assert np.array_equal(O.ref_merge_adapter(m, Ai, Bi, 2.0, -1.0, "f16"), Wi)
+    assert np.array_equal(O.ref_merge_adapter(Wi, Ai, Bi, 0.0, 1.0, "bf16"), Wi)
+
+
 def test_allocator_against_brute_force():
     """ref_alloc / ref_alloc_contiguous / ref_free against the plain definitions:
     the first n free pages in index order; the smallest s with pages s..s+n-1 all

@@ -147,6 +147,63 @@ def test_page_allocator_equals_the_reference_allocator(gpu, tot):
         pa.alloc(pa.can_use_mem_size + 1)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,h_out,rank", [(256, [256, 64, 64, 256], 16), (512, [512] * 4, 64), (128, [128] * 4, 12)])
+def test_merge_and_unmerge_adapter(gpu, dtype, hidden, h_out, rank):
+    """gather_lora_a is the exact transpose-gather; merge_adapter equals the
+    oracle's restatement of the reference within rtol 1e-2 and an absolute term of
+    one storage-type rounding of the update A B * scaling (the reference rounds the
+    update before adding it, the kernel adds the float sum: where W and the update
+    cancel, the difference is that rounding, not a fraction of the result) --
+    1e-3 in fp16, 8e-3 in bf16 at these magnitudes; exactly on integer-valued
+    weights, where merge + unmerge also returns the base weights bit for bit."""
+    from slora_hip.infer_adapter import gather_lora_a, load_rows_into_pool, merge_adapter, unmerge_adapter
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rng = np.random.default_rng(hidden + rank)
+    n_pages, heads = 4 * rank * 3 + 17, 4
+    ranks = [8, rank, 8]
+    a_start, a_len, a_loc = O.build_tables(ranks, rng.permutation(n_pages)[: 4 * sum(ranks)])
+    scal = np.array([1.0, 2.0, 0.5], np.float32)
+    key = torch.zeros((n_pages, heads, hidden // heads), dtype=tdt, device=gpu)
+    val = torch.zeros_like(key)
+    for integer in (False, True):
+        if integer:
+            A = [rng.integers(-2, 3, size=(hidden, rank)).astype(np.float32) for _ in range(4)]
+            Bm = [rng.integers(-2, 3, size=(rank, h_out[p])).astype(np.float32) for p in range(4)]
+            W0 = [rng.integers(-8, 9, size=(hidden, h_out[p])).astype(np.float32) for p in range(4)]
+        else:
+            A = [O.round_to(rng.standard_normal((hidden, rank)).astype(np.float32) / 16, dtype) for _ in range(4)]
+            Bm = [O.round_to(rng.standard_normal((rank, h_out[p])).astype(np.float32) / 4, dtype) for p in range(4)]
+            W0 = [O.round_to(rng.standard_normal((hidden, h_out[p])).astype(np.float32), dtype) for p in range(4)]
+        w = O.pack_w_combined(A, Bm, hidden)
+        loc1 = a_loc[a_start[1]: a_start[1] + a_len[1]]
+        load_rows_into_pool([key, val], [torch.from_numpy(w[0]).to(gpu, tdt).view(4 * rank, heads, -1),
+                                         torch.from_numpy(w[1]).to(gpu, tdt).view(4 * rank, heads, -1)],
+                            torch.from_numpy(loc1).to(gpu))
+        t = [torch.from_numpy(v).to(gpu) for v in (a_start, a_len, a_loc)]
+        scales = torch.from_numpy(scal).to(gpu, torch.float16)
+        for p in range(4):
+            a_p = gather_lora_a(key, t[2], int(a_start[1]) + p * rank, rank, hidden, (rank + 7) // 8 * 8)
+            assert torch.equal(a_p[:, :rank], torch.from_numpy(A[p]).to(gpu, tdt))
+            assert not a_p[:, rank:].any()
+        Wg = [torch.from_numpy(v).to(gpu, tdt) for v in W0]
+        merge_adapter(Wg, key, val, *t, scales, 1)
+        for p in range(4):
+            ref = O.ref_merge_adapter(W0[p], A[p], Bm[p], 2.0, 1.0, dtype)
+            if integer:
+                assert np.array_equal(Wg[p].float().cpu().numpy(), ref), p
+            else:
+                np.testing.assert_allclose(Wg[p].float().cpu().numpy(), ref, rtol=1e-2,
+                                           atol=1e-3 if dtype == "f16" else 8e-3)
+        unmerge_adapter(Wg, key, val, *t, scales, 1)
+        for p in range(4):
+            if integer:
+                assert np.array_equal(Wg[p].float().cpu().numpy(), W0[p]), p
+            else:
+                np.testing.assert_allclose(Wg[p].float().cpu().numpy(), W0[p], rtol=1e-2,
+                                           atol=4e-3 if dtype == "f16" else 3e-2)
+
+
 def test_pool_ops_reject_bad_arguments(gpu):
     from slora_hip.infer_adapter import compact_adapter_tables, launch_var_len_copy, load_rows_into_pool
     buf = torch.zeros((10, 2, 8), dtype=torch.float16, device=gpu)
