@@ -1154,7 +1154,7 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
 }
 
 template <typename T, int NPROJ, bool PLANNED>
-__global__ __launch_bounds__(256, 4) void bgmv_expand_kernel(const ExpandArgs p) {
+__global__ __launch_bounds__(256, 5) void bgmv_expand_kernel(const ExpandArgs p) {
   __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
   expand_body<T, NPROJ, PLANNED, false>(p, (int)blockIdx.x, s_out[threadIdx.x >> 6]);
 }
