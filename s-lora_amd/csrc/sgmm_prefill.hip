@@ -618,10 +618,18 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   blk /= p.n_chunks;
   const int req = blk / p.m_tiles;
   const int m0 = (blk - req * p.m_tiles) * kExpTM;
-  int64_t a;
-  int r, row0, rows;
-  if (!seg_lookup(p.t, req, a, r, row0, rows)) return;
+  // The request's three entries are independent loads: all go out before the first
+  // test, so a workgroup beyond the request's length leaves after one round trip;
+  // the adapter's entries (length, start, scale) are the second round trip.
+  int64_t a = p.t.b_indicies[req];
+  int row0 = p.t.b_start_loc[req];
+  int rows = p.t.b_seq_len[req];
+  asm volatile("" : "+s"(a), "+s"(row0), "+s"(rows));
+  if (row0 < 0 || rows <= 0 || row0 >= p.t.n_tokens) return;
+  if (rows > p.t.n_tokens - row0) rows = p.t.n_tokens - row0;
   if (m0 >= rows) return;
+  if ((uint64_t)a >= (uint64_t)p.t.n_adapters) return;
+  const int r = (int)(p.t.a_len[a] >> 2);
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   if (r_eff <= 0) return;
   const int m_cnt = rows - m0 < kExpTM ? rows - m0 : kExpTM;

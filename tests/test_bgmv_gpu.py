@@ -448,6 +448,69 @@ def test_shrink_and_expand_in_one_launch_equal_the_two_calls(gpu, dtype, hidden,
     assert not slora_hip.plan_wait_timed_out(plan)
 
 
+def test_full_size_s2_properties(gpu, plan_cache_mode):
+    """The benchmark's own configuration (hidden 4096, 200 adapters of ranks
+    {64,32,16,8}, Zipf(1) batch of 256, 65536-page pool), one layer, checked through
+    properties that do not need the CPU oracle at this size:
+    * against torch float32 on the same device from the adapters' unpacked A, B
+      (dense closed form, rtol 1e-2 / atol 1e-3 on the final y with the kernel's
+      own fp16 delta as input of the second product);
+    * doubling every scale doubles y exactly (power of two, zero start) wherever
+      y is a normal fp16 number;
+    * permuting the tokens permutes the results bit for bit (other runs, other
+      workgroups, same sums);
+    * garbage in delta columns beyond an adapter's rank changes nothing."""
+    from slora_hip import dispatch_bgmv, workloads
+    w = workloads.s2_decode(gpu, n_layers=1)
+    B, H, R = w.batch, w.hidden, w.max_rank
+    t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
+    g = torch.Generator(device=gpu)
+    g.manual_seed(5)
+    x = torch.randn((B, H), generator=g, device=gpu).to(w.dtype)
+    key, val = w.key_buffer[0], w.value_buffer[0]
+    perm = torch.randperm(B, generator=g, device=gpu)
+    t_perm = (w.a_start, w.a_len, w.a_loc, w.req_bins[perm].contiguous())
+    ranks_t = torch.from_numpy(w.ranks[w.bins_np]).to(gpu)
+    for p in range(4):
+        d = torch.zeros((B, R), dtype=w.dtype, device=gpu)
+        dispatch_bgmv(d, x, key, *t, p, w.a_scaling)
+        y = torch.zeros((B, H), dtype=w.dtype, device=gpu)
+        dispatch_bgmv(y, d, val, *t, p, w.a_scaling)
+        # dense float32 closed form per adapter in the batch
+        d_ref = torch.zeros((B, R), dtype=torch.float32, device=gpu)
+        y_ref = torch.zeros((B, H), dtype=torch.float32, device=gpu)
+        for a in np.unique(w.bins_np):
+            r = int(w.ranks[a])
+            loc = w.a_loc[int(w.a_start_np[a]) + p * r: int(w.a_start_np[a]) + (p + 1) * r]
+            rows = torch.from_numpy(np.nonzero(w.bins_np == a)[0]).to(gpu)
+            A = key[loc].reshape(r, H).float()                      # [r, H] = A^T
+            Bt = val[loc].reshape(H, r).float()                     # [H, r] = B^T
+            d_ref[rows, :r] = x[rows].float() @ A.t()
+            y_ref[rows] = (d[rows, :r].float() @ Bt.t()) * float(w.scales_np[a])
+        np.testing.assert_allclose(d.float().cpu().numpy(), d_ref.cpu().numpy(), rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(y.float().cpu().numpy(), y_ref.cpu().numpy(), rtol=RTOL, atol=ATOL)
+        # scale x 2  ->  y x 2, exactly
+        y2 = torch.zeros_like(y)
+        dispatch_bgmv(y2, d, val, *t, p, (w.a_scaling * 2).contiguous())
+        normal = y.abs() >= 2.0 ** -13   # below, fp16 is subnormal and rounding does not commute with doubling
+        assert torch.equal(y2[normal], (y * 2)[normal])
+        assert (y2[~normal].float() - 2 * y[~normal].float()).abs().max() <= 2.0 ** -23
+        # token permutation
+        dp = torch.zeros_like(d)
+        dispatch_bgmv(dp, x[perm].contiguous(), key, *t_perm, p, w.a_scaling)
+        assert torch.equal(dp, d[perm])
+        yp = torch.zeros_like(y)
+        dispatch_bgmv(yp, dp, val, *t_perm, p, w.a_scaling)
+        assert torch.equal(yp, y[perm])
+        # columns beyond the rank do not matter
+        dg = d.clone()
+        cols = torch.arange(R, device=gpu)[None, :] >= ranks_t[:, None]
+        dg[cols] = 77.0
+        yg = torch.zeros_like(y)
+        dispatch_bgmv(yg, dg, val, *t, p, w.a_scaling)
+        assert torch.equal(yg, y)
+
+
 def test_plan_is_rejected_for_another_batch_size(gpu):
     import slora_hip
     c = make_case(19, 256, [8, 16], 12, dtype="f16")

@@ -76,6 +76,42 @@ def test_prefill_many_requests(gpu, n_req, lo, hi):
         check(c, g, p, 64, gpu, seed=p)
 
 
+def test_full_size_c3_against_dense_and_decode(gpu):
+    """The C3 configuration itself (bf16, hidden 4096, 64 requests of 8..512 tokens,
+    100 adapters of ranks {64,32,16,8}, 65536-page pool), one layer: shrink and
+    expand against torch float32 on the device from the unpacked A, B (rtol 1e-2;
+    atol 1e-3 for the shrink output, 2e-2 for y, which is a bf16 sum of order-1
+    terms that may cancel), zero-fill of the columns beyond each rank, and rows
+    that belong to no request left alone."""
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand, workloads
+    w, seg = workloads.c3_prefill(gpu, n_layers=1)
+    T, H, R = seg.n_tokens, w.hidden, w.max_rank
+    g = torch.Generator(device=gpu)
+    g.manual_seed(3)
+    x = torch.randn((T + 5, H), generator=g, device=gpu).to(w.dtype)       # 5 rows owned by no request
+    key, val = w.key_buffer[0], w.value_buffer[0]
+    t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
+    starts = np.concatenate([[0], np.cumsum(seg.lens_np)[:-1]])
+    for p in (0, 3):
+        d = torch.full((T + 5, R), 9.0, dtype=w.dtype, device=gpu)
+        lora_get_qkvo_fwd_shrink(x, key.view(-1, H), d, *t, H, p, R, seg.max_len)
+        y0 = torch.randn((T + 5, H), generator=g, device=gpu).to(w.dtype)
+        y = y0.clone()
+        lora_get_qkvo_fwd_expand(d, val.view(-1, H), y, w.a_scaling, *t, H, p, R, seg.max_len)
+        d_ref = torch.zeros((T, R), dtype=torch.float32, device=gpu)
+        y_ref = y0[:T].float().clone()
+        for i, a in enumerate(seg.ids_np):
+            r = int(w.ranks[a])
+            loc = w.a_loc[int(w.a_start_np[a]) + p * r: int(w.a_start_np[a]) + (p + 1) * r]
+            rows = slice(int(starts[i]), int(starts[i]) + int(seg.lens_np[i]))
+            d_ref[rows, :r] = x[rows].float() @ key[loc].reshape(r, H).float().t()
+            y_ref[rows] += (d[rows, :r].float() @ val[loc].reshape(H, r).float().t()) * float(w.scales_np[a])
+        np.testing.assert_allclose(d[:T].float().cpu().numpy(), d_ref.cpu().numpy(), rtol=RTOL, atol=ATOL)
+        np.testing.assert_allclose(y[:T].float().cpu().numpy(), y_ref.cpu().numpy(), rtol=RTOL, atol=2e-2)
+        assert torch.equal(d[T:], torch.full((5, R), 9.0, dtype=w.dtype, device=gpu))
+        assert torch.equal(y[T:], y0[T:])
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_prefill_gather_bit_exact(gpu, dtype):
     rng = np.random.default_rng(5)
