@@ -47,7 +47,14 @@ def _tables(start_indicies, lora_ranks, loc_indicies) -> _cabi.SloraTables:
                              start_indicies.numel(), loc_indicies.numel())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t) -> int:
+    """The current stream of ``t``'s device as a raw handle (the fast private
+    accessor when this torch has it: the public one builds a Stream object)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
