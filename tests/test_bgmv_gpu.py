@@ -448,6 +448,77 @@ def test_shrink_and_expand_in_one_launch_equal_the_two_calls(gpu, dtype, hidden,
     assert not slora_hip.plan_wait_timed_out(plan)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(gpu, seed):
+    """Seeded random shapes: hidden and output widths that are any multiple of 8,
+    ranks that are powers of two, other multiples of 8, or odd, batches from 1 to
+    700, pages wider than the rows, either dtype.  Every way of calling (no plan,
+    plan, q/k/v in one launch, shrink and expand in one launch) against the oracle
+    and against each other bit for bit."""
+    import slora_hip
+    from slora_hip import (dispatch_bgmv, dispatch_bgmv_lora, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_lora,
+                           dispatch_bgmv_qkv_shrink)
+    rng = np.random.default_rng(1000 + seed)
+    hidden = int(rng.integers(1, 129)) * 8 * int(rng.choice([1, 1, 4]))
+    n_ad = int(rng.integers(1, 7))
+    ranks = [int(rng.choice([8, 16, 32, 64, 24, 40, 4, 12, 5, 128])) for _ in range(n_ad)]
+    batch = int(rng.choice([1, 2, 5, 33, 64, 257, 700]))
+    wide = int(rng.choice([1, 1, 2]))
+    h_out = [int(rng.integers(1, 65)) * 8 * wide for _ in range(4)] if rng.random() < 0.5 else None
+    if h_out is not None:
+        h_out = [max(h, max(ranks) + 8) for h in h_out]
+    hidden = max(hidden, max(ranks) + 8)          # shrink means delta narrower than x
+    page_elems = max([hidden] + (h_out or [])) * int(rng.choice([1, 1, 2]))
+    dtype = str(rng.choice(["f16", "bf16"]))
+    c = make_case(2000 + seed, hidden, ranks, batch, dtype=dtype, h_out=h_out, page_elems=page_elems,
+                  zipf_alpha=float(rng.choice([0.0, 1.0, 2.0])))
+    g = GpuCase(c, gpu, heads=1)
+    R = (max(ranks) + 7) // 8 * 8
+    t = (g.a_start, g.a_len, g.a_loc, g.bins)
+    plan = slora_hip.make_plan(*t, R, c.n_pages)
+    y0 = [torch.randn((batch, c.h_out[p]), dtype=g.tdt, device=gpu) for p in range(4)]
+    d_s, y_s = [], []
+    for p in range(4):
+        d = torch.zeros((batch, R), dtype=g.tdt, device=gpu)
+        dispatch_bgmv(d, g.x, g.key, *t, p, g.scales, plan=False)
+        y = y0[p].clone()
+        dispatch_bgmv(y, d, g.value, *t, p, g.scales, plan=False)
+        d_ref, _ = oracle_chain(c, p, R)
+        np.testing.assert_allclose(host(d), d_ref, rtol=RTOL, atol=ATOL)
+        # against the oracle from a zero start (a random start adds a rounding of the sum to
+        # the storage type that cancellation can turn into more than 1 % of the result)
+        yz = torch.zeros_like(y)
+        dispatch_bgmv(yz, d, g.value, *t, p, g.scales, plan=False)
+        y_ref = O.ref_bgmv_expand(np.zeros((batch, c.h_out[p]), np.float32), host(d), c.value, c.a_start, c.a_len,
+                                  c.a_loc, c.bins, p, c.scales, dtype=c.dtype)
+        np.testing.assert_allclose(host(yz), y_ref, rtol=RTOL, atol=ATOL)
+        d_s.append(d)
+        y_s.append(y)
+        d_p = torch.zeros_like(d)
+        dispatch_bgmv(d_p, g.x, g.key, *t, p, g.scales, plan=plan)
+        y_p = y0[p].clone()
+        dispatch_bgmv(y_p, d_p, g.value, *t, p, g.scales, plan=plan)
+        assert torch.equal(d_p, d) and torch.equal(y_p, y), ("planned", p)
+        d_l = torch.zeros_like(d)
+        y_l = y0[p].clone()
+        dispatch_bgmv_lora(y_l, d_l, g.x, g.key, g.value, *t, p, g.scales, plan=plan)
+        assert torch.equal(d_l, d) and torch.equal(y_l, y), ("one launch", p)
+    for planned in (None, plan):
+        kw = {"plan": planned} if planned is not None else {"plan": False}
+        d_f = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+        y_f = [y0[p].clone() for p in range(3)]
+        dispatch_bgmv_qkv_shrink(d_f[0], d_f[1], d_f[2], g.x, g.key, *t, **kw)
+        dispatch_bgmv_qkv_expand(y_f[0], y_f[1], y_f[2], d_f[0], d_f[1], d_f[2], g.value, *t, g.scales, **kw)
+        for p in range(3):
+            assert torch.equal(d_f[p], d_s[p]) and torch.equal(y_f[p], y_s[p]), ("q/k/v", planned is not None, p)
+    d_f = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+    y_f = [y0[p].clone() for p in range(3)]
+    dispatch_bgmv_qkv_lora(y_f[0], y_f[1], y_f[2], d_f[0], d_f[1], d_f[2], g.x, g.key, g.value, *t, g.scales, plan=plan)
+    for p in range(3):
+        assert torch.equal(d_f[p], d_s[p]) and torch.equal(y_f[p], y_s[p]), ("q/k/v one launch", p)
+    assert not slora_hip.plan_wait_timed_out(plan)
+
+
 def test_full_size_s2_properties(gpu, plan_cache_mode):
     """The benchmark's own configuration (hidden 4096, 200 adapters of ranks
     {64,32,16,8}, Zipf(1) batch of 256, 65536-page pool), one layer, checked through

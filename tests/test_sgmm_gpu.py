@@ -76,6 +76,25 @@ def test_prefill_many_requests(gpu, n_req, lo, hi):
         check(c, g, p, 64, gpu, seed=p)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_prefill_random_configurations(gpu, seed):
+    """Seeded random shapes for the segmented kernels: hidden any multiple of 8 up
+    to 4096, ranks of every kind, 1 to 90 requests of 1 to 300 tokens, sorted by
+    adapter or not, either dtype, all four projections against the oracle."""
+    rng = np.random.default_rng(3000 + seed)
+    hidden = int(rng.integers(2, 65)) * 8 * int(rng.choice([1, 2, 8]))
+    ranks = [int(rng.choice([8, 16, 32, 64, 24, 40, 4, 12, 128])) for _ in range(int(rng.integers(1, 6)))]
+    hidden = max(hidden, (max(ranks) + 15) // 8 * 8)
+    n_req = int(rng.choice([1, 3, 17, 90]))
+    hi = int(rng.choice([2, 40, 300]))
+    dtype = str(rng.choice(["f16", "bf16"]))
+    c = seg_case(3100 + seed, hidden, ranks, n_req, 1, hi, dtype, sort=bool(rng.integers(0, 2)))
+    g = GpuCase(c, gpu)
+    R = (max(ranks) + 7) // 8 * 8
+    for p in range(4):
+        check(c, g, p, R, gpu, seed=p)
+
+
 def test_full_size_c3_against_dense_and_decode(gpu):
     """The C3 configuration itself (bf16, hidden 4096, 64 requests of 8..512 tokens,
     100 adapters of ranks {64,32,16,8}, 65536-page pool), one layer: shrink and
