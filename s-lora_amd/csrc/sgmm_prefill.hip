@@ -432,17 +432,21 @@ struct SegExpandArgs {
   int64_t x_stride, w_stride, o_stride;
   int64_t page_elems;
   int scales_dtype;
-  int feat_out, max_rank, qkvo, m_tiles, n_chunks;
+  int feat_out, max_rank, qkvo, m_tiles, m_span, n_chunks;
   int vec_ok;
 };
 
 constexpr int kExpThreads = 256;
-constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, each kExpTMW token rows
-constexpr int kExpMF = 2;                       // 16-row MFMA fragments per wavefront
-constexpr int kExpTMW = 16 * kExpMF;            // token rows per wavefront
-constexpr int kExpTM = kExpTMW * kExpWaves;     // token rows per workgroup
-constexpr int kExpOB = 64;                      // outputs per MFMA block
-constexpr int kExpBlocks = 1;                   // blocks a wavefront walks (512 outputs)
+constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, one 64-output block each
+constexpr int kExpMF = 2;                       // 16-row MFMA fragments per row tile
+constexpr int kExpTMW = 16 * kExpMF;            // token rows per row tile
+constexpr int kExpOB = 64;                      // outputs per wavefront
+constexpr int kExpGroup = kExpOB * kExpWaves;   // outputs per workgroup: 512 contiguous bytes of every row
+#ifndef SLORA_EXP_SPAN_TILES
+#define SLORA_EXP_SPAN_TILES 16
+#endif
+constexpr int kExpSpanTiles = SLORA_EXP_SPAN_TILES;  // most row tiles a workgroup walks
+constexpr int kExpMinGrid = 512;                     // shorter spans rather than fewer workgroups than this
 
 template <typename T>
 __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale, int row0,
@@ -467,10 +471,11 @@ __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t
   }
 }
 
-// One wavefront = kExpTMW token rows x kExpBlocks consecutive 64-output blocks.
-// KS = number of 32-wide K steps that cover the rank (1, 2 or 4).  The delta
-// fragments are loaded once per wavefront; every block then loads its B^T
-// fragments and y values together, multiplies and stores.
+// One wavefront = one 64-output block x a walk over token-row tiles of kExpTMW rows.
+// KS = number of 32-wide K steps that cover the rank (1, 2 or 4).  The B^T
+// fragments of the block are loaded once and stay in registers; every row tile
+// then loads its delta fragments and y values together, multiplies and stores,
+// with the next tile's loads already in flight.
 //
 // MFMA orientation: rows = outputs, columns = tokens, so a lane's C values are
 // consecutive outputs of ONE token row.  The row -> output map
@@ -478,20 +483,45 @@ __device__ void expand_generic(const SegExpandArgs& p, int r, int r_eff, int64_t
 // gives lane group g = m/4 the outputs 8g..8g+7 (tiles 0,1) and 32+8g..32+8g+7
 // (tiles 2,3): each 16-byte access of the four lane groups of a token is one
 // contiguous 64-byte run.
-template <int KS>
-struct ExpandBuf {
-  u32x4 a[4][KS];       // B^T fragments (MFMA A operand)
-  u32x4 y[kExpMF][2];   // y values this lane updates
+//
+// y itself is read and written in another lane order.  In the MFMA order the four
+// lanes of a token cover 64 bytes per instruction, so an instruction touches 16
+// half cache lines; the vector cache handles 8 whole lines per instruction about
+// 1.4x faster.  In the "line order" instruction g covers tokens 8g .. 8g+7 of a
+// fragment, lane (lr, lg) holding 16-byte piece lg + 4*(lr/8) of token 8g + lr%8.
+// Both orders keep a value in the same 16-lane row, at most 8 lanes away, so one
+// DPP move per register converts between them (swap_halves, its own inverse).
+struct ExpandStage {
+  u32x4 y[kExpMF][2];  // y values in line order
 };
 
+// The workgroup's delta rows go through LDS (every wavefront multiplies the same
+// rows): row stride KS*64 + 16 bytes, the pad spreading the 16 rows of an MFMA-order
+// read over all banks.
+template <int KS>
+constexpr int kExpLdsRow = KS * 64 + 16;
+constexpr int kExpChunkRows = 4 * kExpTMW;  // rows staged at a time
+
+// (a, b) in MFMA order [piece lg | piece 4 + lg of token lr]  <->  line order
+// [tokens 0..7 | tokens 8..15, pieces lg + 4*(lr/8)]: a keeps its lanes 0..7 of every 16
+// and takes b's lanes 0..7 into 8..15; b takes a's lanes 8..15 into 0..7 and keeps 8..15.
+__device__ __forceinline__ void swap_halves(u32x4& a, u32x4& b) {
+  constexpr int kRowRor8 = 0x128;  // rotate by 8 inside each row of 16 lanes
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int va = (int)a[q], vb = (int)b[q];
+    a[q] = (uint32_t)__builtin_amdgcn_update_dpp(va, vb, kRowRor8, 0xF, 0xC, false);
+    b[q] = (uint32_t)__builtin_amdgcn_update_dpp(vb, va, kRowRor8, 0xF, 0x3, false);
+  }
+}
+
+// B^T fragments of outputs nb .. nb + 63 (MFMA A operand)
 template <typename T, int KS>
-__device__ __forceinline__ void expand_load(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, int nb,
-                                            const int64_t (&orow)[kExpMF], const bool (&row_ok)[kExpMF], bool live,
-                                            ExpandBuf<KS>& buf) {
+__device__ __forceinline__ void expand_load_weights(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, int nb,
+                                                    u32x4 (&a)[4][KS]) {
   const int lane = threadIdx.x & 63;
   const int lr = lane & 15, lg = lane >> 4;
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
-  const uint16_t* og = reinterpret_cast<const uint16_t*>(p.o);
   const uint32_t page_elems = (uint32_t)p.page_elems;
   // phase 1: every page id (loads back to back, no branch in between)
   int64_t page[4][KS];
@@ -502,7 +532,7 @@ __device__ __forceinline__ void expand_load(const SegExpandArgs& p, int r, int r
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const int d = s * 32 + lg * 8;
-      const bool want = live && n < p.feat_out && d < r_eff && p.t.n_loc > 0;
+      const bool want = n < p.feat_out && d < r_eff && p.t.n_loc > 0;
       const uint32_t flat = (uint32_t)n * (uint32_t)r + (uint32_t)d;
       const uint32_t pg = flat / page_elems;
       off[t][s] = flat - pg * page_elems;
@@ -515,30 +545,85 @@ __device__ __forceinline__ void expand_load(const SegExpandArgs& p, int r, int r
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const bool ok = page[t][s] >= 0;
-      buf.a[t][s] = ldg16(wg + (ok ? page[t][s] * p.w_stride + off[t][s] : 0));
-    }
-#pragma unroll
-  for (int f = 0; f < kExpMF; ++f)
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int n = nb + 32 * h + 8 * lg;
-      const bool ok = live && row_ok[f] && n < p.feat_out;
-      buf.y[f][h] = ldg16(og + orow[f] + (ok ? n : 0));  // a row that is not there repeats row 0 and is never stored
+      a[t][s] = ldg16(wg + (ok ? page[t][s] * p.w_stride + off[t][s] : 0));
     }
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-      if (page[t][s] < 0) buf.a[t][s] = zero16();
+      if (page[t][s] < 0) a[t][s] = zero16();
 }
 
-template <typename T, int KS>
-__device__ __forceinline__ void expand_finish(const SegExpandArgs& p, float scale, int nb,
-                                              const u32x4 (&bfrag)[kExpMF][KS], const int64_t (&orow)[kExpMF],
-                                              const bool (&row_ok)[kExpMF], const ExpandBuf<KS>& buf) {
+// y values of rows m0w .. m0w + kExpTMW - 1 of the request, outputs nb .. nb + 63, in line
+// order; rows at or past m_end read row m_safe instead and are never stored.
+__device__ __forceinline__ void expand_load_rows(const SegExpandArgs& p, int row0, int m0w, int m_end, int m_safe,
+                                                 int nb, ExpandStage& st) {
   const int lane = threadIdx.x & 63;
-  const int lg = lane >> 4;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint16_t* og = reinterpret_cast<const uint16_t*>(p.o);
+  const int n_line = nb + 8 * (lg + 4 * (lr >> 3));
+#pragma unroll
+  for (int f = 0; f < kExpMF; ++f)
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int m = m0w + f * 16 + 8 * g + (lr & 7);
+      const int64_t row = row0 + (m < m_end ? m : m_safe);
+      st.y[f][g] = ldg16(og + row * p.o_stride + (n_line < p.feat_out ? n_line : 0));
+    }
+}
+
+// Delta rows of one chunk (kExpChunkRows rows from m_chunk; rows at or past m_end repeat
+// row m_safe) as the whole workgroup loads them: an instruction covers whole 128-byte
+// lines, lane t of the workgroup takes pieces t, t + 256, ...
+template <int KS>
+struct ExpandChunk {
+  u32x4 v[KS * 2];  // kExpChunkRows * KS * 4 pieces / kExpThreads
+};
+
+template <int KS>
+__device__ __forceinline__ void expand_chunk_load(const SegExpandArgs& p, int row0, int m_chunk, int m_end, int m_safe,
+                                                  ExpandChunk<KS>& c) {
+  constexpr int kPieces = KS * 4;  // 16-byte pieces of a row
+  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
+#pragma unroll
+  for (int u = 0; u < KS * 2; ++u) {
+    const int idx = (int)threadIdx.x + u * kExpThreads;
+    const int row = idx / kPieces, d = (idx - row * kPieces) * 8;
+    const int m = m_chunk + row;
+    // columns at or past max_rank may not exist in the row; the fragments zero them anyway
+    c.v[u] = ldg16(xg + (int64_t)(row0 + (m < m_end ? m : m_safe)) * p.x_stride + (d < p.max_rank ? d : 0));
+  }
+}
+
+template <int KS>
+__device__ __forceinline__ void expand_chunk_store(const ExpandChunk<KS>& c, char* s_chunk) {
+  constexpr int kPieces = KS * 4;
+#pragma unroll
+  for (int u = 0; u < KS * 2; ++u) {
+    const int idx = (int)threadIdx.x + u * kExpThreads;
+    const int row = idx / kPieces, piece = idx - row * kPieces;
+    *reinterpret_cast<u32x4*>(s_chunk + row * kExpLdsRow<KS> + piece * 16) = c.v[u];
+  }
+}
+
+// One row tile: multiply the staged delta rows m_rel .. m_rel + 31 of the span by the
+// block's B^T fragments, add to y and store.
+template <typename T, int KS>
+__device__ __forceinline__ void expand_finish(const SegExpandArgs& p, float scale, int r_eff, int row0, int m0w,
+                                              int m_end, int nb, const u32x4 (&a)[4][KS], const char* s_tile,
+                                              const ExpandStage& st) {
+  const int lane = threadIdx.x & 63;
+  const int lr = lane & 15, lg = lane >> 4;
   uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
+  // delta fragments (MFMA B operand) in MFMA order, zero past the adapter's rank
+  u32x4 b[kExpMF][KS];
+#pragma unroll
+  for (int f = 0; f < kExpMF; ++f)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      b[f][s] = *reinterpret_cast<const u32x4*>(s_tile + (f * 16 + lr) * kExpLdsRow<KS> + s * 64 + lg * 16);
+      if (s * 32 + lg * 8 >= r_eff) b[f][s] = zero16();
+    }
   f32x4 acc[kExpMF][4];
 #pragma unroll
   for (int f = 0; f < kExpMF; ++f)
@@ -546,78 +631,93 @@ __device__ __forceinline__ void expand_finish(const SegExpandArgs& p, float scal
     for (int t = 0; t < 4; ++t) {
       acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(buf.a[t][s], bfrag[f][s], acc[f][t]);
+      for (int s = 0; s < KS; ++s) acc[f][t] = mfma16<T>(a[t][s], b[f][s], acc[f][t]);
     }
   // C tile t: lane holds token column lr, rows 4*lg + i  ->  output 32*(t/2) + 8*lg + 4*(t%2) + i
+  const int n_line = nb + 8 * (lg + 4 * (lr >> 3));
 #pragma unroll
   for (int f = 0; f < kExpMF; ++f) {
+    u32x4 y0 = st.y[f][0], y1 = st.y[f][1];
+    swap_halves(y0, y1);  // line order -> MFMA order: y0 = outputs nb + 8*lg .., y1 = outputs nb + 32 + 8*lg ..
+    u32x4 out[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int n = nb + 32 * h + 8 * lg;
-      if (row_ok[f] && n < p.feat_out) {
-        u32x4 out;
+      const u32x4& yv = h == 0 ? y0 : y1;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          // outputs n + 2q, n + 2q + 1  <-  tile 2h + (2q)/4, element (2q)%4 and the next
-          const int e0 = 2 * q;
-          const float d0 = acc[f][2 * h + (e0 >> 2)][e0 & 3] * scale;
-          const float d1 = acc[f][2 * h + ((e0 + 1) >> 2)][(e0 + 1) & 3] * scale;
-          const uint16_t lo = T::from_float(T::lo(buf.y[f][h][q]) + d0);
-          const uint16_t hi = T::from_float(T::hi(buf.y[f][h][q]) + d1);
-          out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
-        }
-        *reinterpret_cast<u32x4*>(og + orow[f] + n) = out;
+      for (int q = 0; q < 4; ++q) {
+        // outputs n + 2q, n + 2q + 1  <-  tile 2h + (2q)/4, element (2q)%4 and the next
+        const int e0 = 2 * q;
+        const float d0 = acc[f][2 * h + (e0 >> 2)][e0 & 3] * scale;
+        const float d1 = acc[f][2 * h + ((e0 + 1) >> 2)][(e0 + 1) & 3] * scale;
+        const uint16_t lo = T::from_float(T::lo(yv[q]) + d0);
+        const uint16_t hi = T::from_float(T::hi(yv[q]) + d1);
+        out[h][q] = (uint32_t)lo | ((uint32_t)hi << 16);
       }
     }
-  }
-}
-
-template <typename T, int KS>
-__device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
-                                            int row0, int m0w, int m_cnt_w, int n0, int n_end) {
-  const int lane = threadIdx.x & 63;
-  const int lr = lane & 15, lg = lane >> 4;
-  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
-  // MFMA B operand: this wavefront's token rows x rank, kept for all blocks
-  u32x4 bfrag[kExpMF][KS];
-  int64_t orow[kExpMF];
-  bool row_ok[kExpMF];
+    swap_halves(out[0], out[1]);  // back to line order
 #pragma unroll
-  for (int f = 0; f < kExpMF; ++f) {
-    const int m = f * 16 + lr;
-    row_ok[f] = m < m_cnt_w;
-    const int64_t row = row0 + m0w + (row_ok[f] ? m : 0);
-    orow[f] = row * p.o_stride;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      const int d = s * 32 + lg * 8;
-      bfrag[f][s] = (row_ok[f] && d < r_eff) ? ldg16(xg + row * p.x_stride + d) : zero16();
+    for (int g = 0; g < 2; ++g) {
+      const int m = m0w + f * 16 + 8 * g + (lr & 7);
+      if (m < m_end && n_line < p.feat_out)
+        *reinterpret_cast<u32x4*>(og + (int64_t)(row0 + m) * p.o_stride + n_line) = out[g];
     }
   }
-  // One buffer: the loop is not unrolled, the other wavefronts of the CU cover
-  // the two round trips (page ids, then fragments) of every block.
+}
+
+// The whole workgroup enters and stays to the end: the delta rows go through LDS in
+// chunks of kExpChunkRows rows, two buffers, one barrier per chunk.  Between barriers
+// the wavefront walks the chunk's row tiles for its own outputs nb .. nb + 63, the
+// next tile's y values and the next chunk's delta rows always in flight.
+template <typename T, int KS>
+__device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r_eff, int64_t base_li, float scale,
+                                            int row0, int m0, int m_end, int nb, char* s_x) {
+  constexpr int kChunkBytes = kExpChunkRows * kExpLdsRow<KS>;
+  const bool live = nb < p.feat_out;  // a wavefront past the last output only helps with the staging
+  u32x4 a[4][KS];
+  ExpandStage cur;
+  ExpandChunk<KS> chunk;
+  // in program order: the first y values and delta rows (they need nothing but the
+  // row), then the B^T fragments behind their page ids
+  expand_load_rows(p, row0, m0, m_end, m0, nb, cur);
+  expand_chunk_load<KS>(p, row0, m0, m_end, m0, chunk);
+  expand_load_weights<T, KS>(p, r, r_eff, base_li, live ? nb : 0, a);
+  expand_chunk_store<KS>(chunk, s_x);
+  __syncthreads();
+  int buf = 0;
 #pragma unroll 1
-  for (int nb = n0; nb < n_end; nb += kExpOB) {
-    ExpandBuf<KS> buf;
-    expand_load<T, KS>(p, r, r_eff, base_li, nb, orow, row_ok, true, buf);
-    expand_finish<T, KS>(p, scale, nb, bfrag, orow, row_ok, buf);
+  for (int mc = m0; mc < m_end; mc += kExpChunkRows) {
+    expand_chunk_load<KS>(p, row0, mc + kExpChunkRows, m_end, m0, chunk);
+    if (live) {
+#pragma unroll 1
+      for (int m0w = mc; m0w < mc + kExpChunkRows && m0w < m_end; m0w += kExpTMW) {
+        ExpandStage nxt;  // past the end every lane re-reads row m0; nothing of it is stored
+        expand_load_rows(p, row0, m0w + kExpTMW, m_end, m0, nb, nxt);
+        expand_finish<T, KS>(p, scale, r_eff, row0, m0w, m_end, nb, a,
+                             s_x + buf * kChunkBytes + (m0w - mc) * kExpLdsRow<KS>, cur);
+        cur = nxt;
+      }
+    }
+    buf ^= 1;
+    expand_chunk_store<KS>(chunk, s_x + buf * kChunkBytes);  // last read two barriers ago
+    __syncthreads();
   }
 }
 
-// Workgroup = (request, tile of 4 * kExpTMW tokens, super-block of kExpBlocks * 64
-// outputs): its 4 wavefronts take kExpTMW token rows each and share the B^T
-// fragments through the CU's L1.
+// Workgroup = (request, span of p.m_span token rows, group of 256 outputs): wavefront
+// w takes the group's w-th block of 64 outputs, keeps that block's B^T fragments
+// and walks the span's row tiles, so the four wavefronts together read and write
+// 512 contiguous bytes of every row.
 template <typename T, int KS>
 __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p) {
   const int wave = threadIdx.x >> 6;
-  // the output super-block is the fastest index: consecutive workgroup ids go to
+  // the output group is the fastest index: consecutive workgroup ids go to
   // the 8 XCDs in turn, so every XCD owns 1/8 of the output columns of ALL
   // requests -- disjoint pieces of B^T per L2 and an even share of the y traffic
   int blk = blockIdx.x;
-  const int chunk = blk % p.n_chunks;
+  const int group = blk % p.n_chunks;
   blk /= p.n_chunks;
   const int req = blk / p.m_tiles;
-  const int m0 = (blk - req * p.m_tiles) * kExpTM;
+  const int m0 = (blk - req * p.m_tiles) * p.m_span;
   // The request's three entries are independent loads: all go out before the first
   // test, so a workgroup beyond the request's length leaves after one round trip;
   // the adapter's entries (length, start, scale) are the second round trip.
@@ -632,21 +732,20 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   const int r = (int)(p.t.a_len[a] >> 2);
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   if (r_eff <= 0) return;
-  const int m_cnt = rows - m0 < kExpTM ? rows - m0 : kExpTM;
-  const int n0 = chunk * (kExpOB * kExpBlocks);
-  const int n_end = n0 + kExpOB * kExpBlocks < p.feat_out ? n0 + kExpOB * kExpBlocks : p.feat_out;
+  const int m_end = rows - m0 < p.m_span ? rows : m0 + p.m_span;
   const int64_t base_li = p.t.a_start[a] + (int64_t)r * p.qkvo;
   const float scale = load_scale(p.scales, p.scales_dtype, a);
   if (!p.vec_ok || (r & 7) != 0 || (r_eff & 7) != 0 || r_eff > 128) {
-    expand_generic<T>(p, r, r_eff, base_li, scale, row0, m0, m_cnt, n0, n_end - n0);
+    const int n0 = group * kExpGroup;
+    const int n_end = n0 + kExpGroup < p.feat_out ? n0 + kExpGroup : p.feat_out;
+    expand_generic<T>(p, r, r_eff, base_li, scale, row0, m0, m_end - m0, n0, n_end - n0);
     return;
   }
-  const int m0w = m0 + wave * kExpTMW;
-  if (m0w >= rows) return;
-  const int m_cnt_w = rows - m0w < kExpTMW ? rows - m0w : kExpTMW;
+  const int nb = group * kExpGroup + wave * kExpOB;
   // KS 32-wide steps cover max_rank (chosen on the host); a smaller adapter
   // rank leaves the upper fragments zero
-  expand_mfma<T, KS>(p, r, r_eff, base_li, scale, row0, m0w, m_cnt_w, n0, n_end);
+  extern __shared__ __align__(16) char s_delta[];
+  expand_mfma<T, KS>(p, r, r_eff, base_li, scale, row0, m0, m_end, nb, s_delta);
 }
 
 // ---------------------------------------------------------------------------
@@ -697,18 +796,31 @@ int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
+template <typename T, int KS>
+int launch_seg_expand_ks(const SegExpandArgs& p, int64_t grid, hipStream_t stream) {
+  auto kernel = sgmm_expand_kernel<T, KS>;
+  constexpr int lds = 2 * kExpChunkRows * kExpLdsRow<KS>;  // 68 KiB for ranks up to 128
+  static bool attr_done = lds <= 64 * 1024;  // benign if two threads race: the call is idempotent
+  if (!attr_done) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return SLORA_ERR_LAUNCH;
+    }
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kExpThreads), lds, stream, p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
 template <typename T>
 int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
   const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles * p.n_chunks;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  if (p.max_rank <= 32)
-    hipLaunchKernelGGL((sgmm_expand_kernel<T, 1>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
-  else if (p.max_rank <= 64)
-    hipLaunchKernelGGL((sgmm_expand_kernel<T, 2>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
-  else
-    hipLaunchKernelGGL((sgmm_expand_kernel<T, 4>), dim3((uint32_t)grid), dim3(kExpThreads), 0, stream, p);
-  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+  if (p.max_rank <= 32) return launch_seg_expand_ks<T, 1>(p, grid, stream);
+  if (p.max_rank <= 64) return launch_seg_expand_ks<T, 2>(p, grid, stream);
+  return launch_seg_expand_ks<T, 4>(p, grid, stream);
 }
 
 }  // namespace
@@ -784,8 +896,14 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
   p.feat_out = (int)feat_out;
   p.max_rank = (int)max_rank;
   p.qkvo = qkvo;
-  p.m_tiles = (int)((max_input_len + kExpTM - 1) / kExpTM);
-  p.n_chunks = (int)((feat_out + kExpOB * kExpBlocks - 1) / (kExpOB * kExpBlocks));
+  p.n_chunks = (int)((feat_out + kExpGroup - 1) / kExpGroup);
+  // rows a workgroup walks: up to kExpSpanTiles tiles, fewer while that leaves the chip short of workgroups
+  int64_t tiles = kExpSpanTiles;
+  while (tiles > 1 &&
+         n_requests * ((max_input_len + kExpTMW * tiles - 1) / (kExpTMW * tiles)) * p.n_chunks < kExpMinGrid)
+    tiles >>= 1;
+  p.m_span = (int)(kExpTMW * tiles);
+  p.m_tiles = (int)((max_input_len + p.m_span - 1) / p.m_span);
   p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
              (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
