@@ -92,7 +92,7 @@ struct SegShrinkArgs {
 #endif
 };
 
-constexpr int kShrThreads = 512;
+constexpr int kShrThreads = 256;
 constexpr int kShrWaves = kShrThreads / kWave;  // K is split over the 8 wavefronts
 constexpr int kShrMF = 4;                       // 16-row A fragments per tile
 constexpr int kShrTM = 16 * kShrMF;             // token rows per tile
@@ -121,56 +121,87 @@ __device__ void shrink_generic(const SegShrinkArgs& p, int r_eff, int64_t base_l
   }
 }
 
-// One wavefront's share of the K loop of a 32-token x (16 * NT)-rank tile.  Its K
-// steps (32 k each) come in adjacent pairs -- global step (i / 2) * 16 + 2 * wave +
-// (i & 1) -- so the two halves of a 128-byte line are read back to back by the same
-// wavefront.  The loads of one step are in flight while the previous one is
-// multiplied; two workgroups share a compute unit (128 registers per lane), so one
-// can stream while the other looks up its pages or reduces its partial sums.  No load sits inside a branch (the wait
-// counters then stay exact): the main loop only runs where all of its steps exist,
-// and the tail re-reads the last step where one does not.
+// Two lane orders of a 16-row x 64-k block (two MFMA K steps, one 128-byte line per row).
+// MFMA order: register s (K step s) of lane (lr, lg) holds row lr, 16-byte piece 4*s + lg.
+// Line order: register g holds row 8*g + lr%8, piece lg + 4*(lr/8) -- one load instruction
+// covers 8 whole lines instead of 16 half lines, which the vector cache serves about 1.4x
+// faster.  Both orders keep a value inside its 16-lane row, at most 8 lanes away: one DPP
+// move per register converts between them, and the conversion is its own inverse.
+__device__ __forceinline__ void swap_halves(u32x4& a, u32x4& b) {
+  constexpr int kRowRor8 = 0x128;  // rotate by 8 inside each row of 16 lanes
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int va = (int)a[q], vb = (int)b[q];
+    // a keeps its lanes 0..7 of every 16 and takes b's lanes 0..7 into 8..15;
+    // b takes a's lanes 8..15 into 0..7 and keeps its lanes 8..15
+    a[q] = (uint32_t)__builtin_amdgcn_update_dpp(va, vb, kRowRor8, 0xF, 0xC, false);
+    b[q] = (uint32_t)__builtin_amdgcn_update_dpp(vb, va, kRowRor8, 0xF, 0x3, false);
+  }
+}
+
+// One wavefront's share of the K loop of a 64-token x (16 * NT)-rank tile: the
+// 64-k blocks wave, wave + 8, ...  A block's fragments are loaded in line order
+// (xline / wline: the rows of the lane's two loads per fragment) and converted when
+// they are multiplied; the loads of one block are in flight while the previous one
+// is multiplied.  No load sits inside a branch (the wait counters then stay
+// exact): the main loop only runs where all of its blocks exist, and the tail
+// re-reads the last block where one does not.
 template <typename T, int NT>
-__device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xrow)[kShrMF], const uint16_t* const (&wrow)[4],
-                                              int ksteps, int wave, int lg, int h_in, f32x4 (&acc)[kShrMF][4]) {
-  const int full = ksteps / (2 * kShrWaves), extra = ksteps - full * 2 * kShrWaves - 2 * wave;
-  const int n = 2 * full + (extra <= 0 ? 0 : (extra >= 2 ? 2 : 1));  // steps of this wavefront
-  if (n == 0) return;
-  const bool ragged_k = (h_in & 31) != 0;
-  auto load_step = [&](int i, u32x4 (&af)[kShrMF], u32x4 (&bf)[NT]) {
+__device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kShrMF][2],
+                                              const uint16_t* const (&wline)[4][2], int wave, int piece, int h_in,
+                                              f32x4 (&acc)[kShrMF][4]) {
+  const int blocks = (h_in + 63) >> 6;
+  const int n = (blocks - wave + kShrWaves - 1) / kShrWaves;  // blocks of this wavefront
+  if (n <= 0) return;
+  const bool ragged_k = (h_in & 63) != 0;
+  struct Block {
+    u32x4 a[kShrMF][2], b[NT][2];
+  };
+  auto load_block = [&](int i, Block& blk) {
     if (i >= n) i = n - 1;
-    int k = ((i >> 1) * (2 * kShrWaves) + 2 * wave + (i & 1)) * 32 + lg * 8;
+    int k = (i * kShrWaves + wave) * 64 + piece * 8;
     const bool k_in = k < h_in;
     if (!k_in) k = 0;
 #pragma unroll
-    for (int f = 0; f < kShrMF; ++f) af[f] = ldg16(xrow[f] + k);
+    for (int f = 0; f < kShrMF; ++f)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) bf[t] = ldg16(wrow[t] + k);
-    if (ragged_k && !k_in) {
-#pragma unroll
-      for (int f = 0; f < kShrMF; ++f) af[f] = zero16();
-#pragma unroll
-      for (int t = 0; t < NT; ++t) bf[t] = zero16();
-    }
-  };
-  auto mul_step = [&](const u32x4 (&af)[kShrMF], const u32x4 (&bf)[NT]) {
+      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16(xline[f][g] + k);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int f = 0; f < kShrMF; ++f) acc[f][t] = mfma16<T>(af[f], bf[t], acc[f][t]);
+      for (int g = 0; g < 2; ++g) blk.b[t][g] = ldg16(wline[t][g] + k);
+    if (ragged_k && !k_in) {
+#pragma unroll
+      for (int f = 0; f < kShrMF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) blk.b[t][0] = blk.b[t][1] = zero16();
+    }
   };
-  u32x4 a0[kShrMF], b0[NT], a1[kShrMF], b1[NT];
-  load_step(0, a0, b0);
+  auto mul_block = [&](Block& blk) {
+#pragma unroll
+    for (int f = 0; f < kShrMF; ++f) swap_halves(blk.a[f][0], blk.a[f][1]);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) swap_halves(blk.b[t][0], blk.b[t][1]);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int f = 0; f < kShrMF; ++f) acc[f][t] = mfma16<T>(blk.a[f][s], blk.b[t][s], acc[f][t]);
+  };
+  Block c0, c1;
+  load_block(0, c0);
   int i = 0;
   for (; i + 2 < n; i += 2) {
-    load_step(i + 1, a1, b1);
-    mul_step(a0, b0);
-    load_step(i + 2, a0, b0);
-    mul_step(a1, b1);
+    load_block(i + 1, c1);
+    mul_block(c0);
+    load_block(i + 2, c0);
+    mul_block(c1);
   }
-  // one or two steps are left; step i is loaded
-  load_step(i + 1, a1, b1);
-  mul_step(a0, b0);
-  if (i + 1 < n) mul_step(a1, b1);
+  // one or two blocks are left; block i is loaded
+  load_block(i + 1, c1);
+  mul_block(c0);
+  if (i + 1 < n) mul_block(c1);
 }
 
 // One tile: token rows row_first .. row_first + m_cnt (m_cnt <= kShrTM) of a request
@@ -184,35 +215,41 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
   uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
-  const int lr = lane & 15, lg = lane >> 4;  // fragment row / k-group of this lane
-  const int ksteps = (p.h_in + 31) >> 5;     // 32 k per MFMA
+  const int lr = lane & 15, lg = lane >> 4;  // MFMA order: fragment row / k-group of this lane
+  const int lrow = lr & 7, piece = lg + 4 * (lr >> 3);  // line order: row inside a half fragment, 16-byte piece
 
-  // token rows of the two A fragments (clamped; rows past the end contribute
-  // nothing because their results are never stored)
-  const uint16_t* xrow[kShrMF];
+  // token rows of the lane's two loads per A fragment (clamped; rows past the end
+  // contribute nothing because their results are never stored)
+  const uint16_t* xline[kShrMF][2];
 #pragma unroll
-  for (int f = 0; f < kShrMF; ++f) {
-    int m = f * 16 + lr;
-    if (m >= m_cnt) m = m_cnt - 1;
-    xrow[f] = xg + (row_first + m) * p.x_stride;
-  }
+  for (int f = 0; f < kShrMF; ++f)
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      int m = f * 16 + 8 * g + lrow;
+      if (m >= m_cnt) m = m_cnt - 1;
+      xline[f][g] = xg + (row_first + m) * p.x_stride;
+    }
 
   for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
     const int nb_cnt = p.max_rank - nb0 < kShrNB ? p.max_rank - nb0 : kShrNB;
     if (nb0 < r_eff) {
-      // weight rows of the four B fragments: the four page lookups go out together;
-      // a row that does not exist (j >= r_eff, bad page id) reads pool page 0 --
-      // its products only reach output columns that are zeroed below
-      const uint16_t* wrow[4];
+      // weight rows of the lane's two loads per B fragment: the page lookups go out
+      // together; a row that does not exist (j >= r_eff, bad page id) reads pool page
+      // 0 -- its products only reach output columns that are zeroed below
+      const uint16_t* wline[4][2];
       {
-        int64_t pg[4];
+        int64_t pg[4][2];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int j = nb0 + t * 16 + lr;
-          pg[t] = seg_page_nobranch(p.t, base_li + j, j < r_eff && p.t.n_loc > 0);
-        }
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) wrow[t] = wg + (pg[t] >= 0 ? pg[t] : 0) * p.w_stride;
+          for (int g = 0; g < 2; ++g) {
+            const int j = nb0 + t * 16 + 8 * g + lrow;
+            pg[t][g] = seg_page_nobranch(p.t, base_li + j, j < r_eff && p.t.n_loc > 0);
+          }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int g = 0; g < 2; ++g) wline[t][g] = wg + (pg[t][g] >= 0 ? pg[t][g] : 0) * p.w_stride;
       }
       const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
       f32x4 acc[kShrMF][4];
@@ -222,10 +259,10 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
         for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
       switch (n_tiles) {
-        case 1: shrink_k_loop<T, 1>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
-        case 2: shrink_k_loop<T, 2>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
-        case 3: shrink_k_loop<T, 3>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
-        default: shrink_k_loop<T, 4>(xrow, wrow, ksteps, wave, lg, p.h_in, acc); break;
+        case 1: shrink_k_loop<T, 1>(xline, wline, wave, piece, p.h_in, acc); break;
+        case 2: shrink_k_loop<T, 2>(xline, wline, wave, piece, p.h_in, acc); break;
+        case 3: shrink_k_loop<T, 3>(xline, wline, wave, piece, p.h_in, acc); break;
+        default: shrink_k_loop<T, 4>(xline, wline, wave, piece, p.h_in, acc); break;
       }
       // C tile: lane holds column lr, rows 4*lg + i
       float* mine = s_part + wave * (kShrTM * kShrLd);
@@ -291,7 +328,7 @@ __device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave,
 // whatever the mix of request lengths and ranks.  A workgroup owns the units
 // whose start falls into its part and walks them as tiles of up to kShrMF units.
 template <typename T>
-__global__ __launch_bounds__(kShrThreads, 2) void sgmm_shrink_kernel(const SegShrinkArgs p) {
+__global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   __shared__ int64_t s_wave[kShrWaves];
   __shared__ int s_row0[kShrChunk], s_rows[kShrChunk], s_ub[kShrChunk], s_ue[kShrChunk], s_rank[kShrChunk];
@@ -501,19 +538,6 @@ struct ExpandStage {
 template <int KS>
 constexpr int kExpLdsRow = KS * 64 + 16;
 constexpr int kExpChunkRows = 4 * kExpTMW;  // rows staged at a time
-
-// (a, b) in MFMA order [piece lg | piece 4 + lg of token lr]  <->  line order
-// [tokens 0..7 | tokens 8..15, pieces lg + 4*(lr/8)]: a keeps its lanes 0..7 of every 16
-// and takes b's lanes 0..7 into 8..15; b takes a's lanes 8..15 into 0..7 and keeps 8..15.
-__device__ __forceinline__ void swap_halves(u32x4& a, u32x4& b) {
-  constexpr int kRowRor8 = 0x128;  // rotate by 8 inside each row of 16 lanes
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int va = (int)a[q], vb = (int)b[q];
-    a[q] = (uint32_t)__builtin_amdgcn_update_dpp(va, vb, kRowRor8, 0xF, 0xC, false);
-    b[q] = (uint32_t)__builtin_amdgcn_update_dpp(vb, va, kRowRor8, 0xF, 0x3, false);
-  }
-}
 
 // B^T fragments of outputs nb .. nb + 63 (MFMA A operand)
 template <typename T, int KS>
