@@ -317,6 +317,34 @@ __device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave,
   return before + inc;
 }
 
+// Cost of walking `units` 16-row units of a rank-r request as tiles of up to kShrMF units, in
+// eighths of what a weight row costs: measured per tile 6.7 us + 0.2 us per weight row, plus
+// 0.177 us per activation row (hidden 4096; all three scale alike with the hidden size).
+// 32-bit: callers keep units below 2^16.
+constexpr uint32_t kShrCostUnit = 7 * kShrUnit;
+__device__ __forceinline__ uint32_t shrink_tile_cost(int r_eff) { return 268u + 8u * (uint32_t)r_eff; }
+__device__ __forceinline__ uint32_t shrink_chunk_cost(int units, int r_eff) {
+  const uint32_t tiles = ((uint32_t)units + kShrMF - 1) / kShrMF;
+  return tiles * shrink_tile_cost(r_eff) + (uint32_t)units * kShrCostUnit;
+}
+
+// About the fewest even chunks of a request of `units` units such that none costs more than
+// t.  Float arithmetic (a chain of exact integer divisions costs microseconds on a lone
+// wavefront): the count only steers the balance, and every wavefront computes the same one.
+__device__ __forceinline__ int shrink_chunks_needed(int units, int r_eff, uint32_t t) {
+  // largest chunk: m whole tiles, then e more units of one more tile
+  const float a = (float)shrink_tile_cost(r_eff), full = a + (float)(kShrMF * kShrCostUnit);
+  const float m = __builtin_floorf((float)t * __builtin_amdgcn_rcpf(full));
+  const float rem = (float)t - m * full;
+  float e = __builtin_floorf((rem - a) * (1.0f / (float)kShrCostUnit));
+  e = e < 0.f ? 0.f : (e > (float)(kShrMF - 1) ? (float)(kShrMF - 1) : e);
+  float size = m * (float)kShrMF + e;
+  if (!(size >= 1.f)) return units;
+  if (size > (float)units) size = (float)units;
+  int n = (int)__builtin_ceilf((float)units * __builtin_amdgcn_rcpf(size));
+  return n < 1 ? 1 : (n > units ? units : n);
+}
+
 // The requests are cut into units of 16 token rows, a unit of a rank-r request
 // costing kShrTM + r: its share of the bytes a full tile moves -- 16 activation
 // rows and a quarter of the r weight rows (a weight row measures as costly as an
@@ -379,23 +407,28 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
       total += tot;
     }
   }
+  // Few requests: no workgroup is given rows of two requests (each would cost it a tile's
+  // fixed share); request j is cut into n_j even chunks, one workgroup each.
+  const bool aligned = p.t.n_requests <= kShrChunk && p.t.n_requests <= parts && p.m_tiles < (1 << 14);
   int64_t carry = 0;  // cost in front of the current chunk of requests
   for (int c0 = 0; c0 < p.t.n_requests; c0 += kShrChunk) {
     int64_t base_li = 0;
     int r = 0, row0 = 0, rows = 0, units = 0;
     const int64_t cu = describe(c0 + tid, base_li, r, row0, rows, units);
     int64_t tot = 0;
-    const int64_t cp = carry + shrink_block_scan(cu * units, s_wave, &tot) - cu * units;  // cost in front of me
-    if (p.t.n_requests <= kShrChunk) total = tot;
-    if (total <= 0) return;
-    const int64_t lo = total * part / parts, hi = total * (part + 1) / parts;
-    // units of my request whose start cost cp + u * cu lies in [lo, hi)
     int ub = 0, ue = 0;
-    if (units > 0) {
-      const int64_t b = lo > cp ? (lo - cp + cu - 1) / cu : 0;
-      const int64_t e = hi > cp ? (hi - cp + cu - 1) / cu : 0;
-      ub = b < units ? (int)b : units;
-      ue = e < units ? (int)e : units;
+    if (!aligned) {
+      const int64_t cp = carry + shrink_block_scan(cu * units, s_wave, &tot) - cu * units;  // cost in front of me
+      if (p.t.n_requests <= kShrChunk) total = tot;
+      if (total <= 0) return;
+      if (units > 0) {
+        // units of my request whose start cost cp + u * cu lies in [lo, hi)
+        const int64_t lo = total * part / parts, hi = total * (part + 1) / parts;
+        const int64_t b = lo > cp ? (lo - cp + cu - 1) / cu : 0;
+        const int64_t e = hi > cp ? (hi - cp + cu - 1) / cu : 0;
+        ub = b < units ? (int)b : units;
+        ue = e < units ? (int)e : units;
+      }
     }
     if (tid == 0) {
       s_first = kShrChunk;
@@ -406,7 +439,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
       s_ub[tid] = ub;
       s_ue[tid] = ue;
       s_row0[tid] = row0;
-      s_rows[tid] = rows;
+      s_rows[tid] = units > 0 ? rows : 0;
       s_rank[tid] = r;
       s_base[tid] = base_li;
       if (ue > ub) {
@@ -415,6 +448,87 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
       }
     }
     __syncthreads();
+    if (aligned) {
+      // Every wavefront repeats the search on its own (shuffles only, no barrier): lane
+      // l looks after requests l, l + 64, ...  T, the cost of the dearest chunk, is
+      // bisected down to the least value whose n_j still sum to at most the grid
+      // (8 rounds: 1/256 of the range).
+      constexpr int kPerLane = kShrChunk / kWave;
+      const int lane = tid & 63;
+      int un[kPerLane], re[kPerLane];
+      uint32_t t_hi = 0;  // one chunk per request always fits: n_requests <= parts
+      uint32_t t_sum = 0;
+#pragma unroll
+      for (int q = 0; q < kPerLane; ++q) {
+        const int idx = lane + q * kWave;
+        un[q] = (s_rows[idx] + kShrUnit - 1) / kShrUnit;
+        re[q] = s_rank[idx] < p.max_rank ? s_rank[idx] : p.max_rank;
+        if (idx >= p.t.n_requests) un[q] = 0;
+        const uint32_t c = un[q] > 0 ? shrink_chunk_cost(un[q], re[q]) : 0u;
+        t_hi = c > t_hi ? c : t_hi;
+        t_sum += c;
+      }
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)t_hi, o, kWave);
+        t_hi = other > t_hi ? other : t_hi;
+        t_sum += (uint32_t)__shfl_xor((int)t_sum, o, kWave);
+      }
+      uint32_t t_lo = 0;  // infeasible (or untested) bound
+      auto fits = [&](uint32_t t) {
+        int sum = 0;
+#pragma unroll
+        for (int q = 0; q < kPerLane; ++q)
+          if (q * kWave < p.t.n_requests) sum += un[q] > 0 ? shrink_chunks_needed(un[q], re[q], t) : 0;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+        return sum <= parts;
+      };
+      // The even share is a lower bound (cutting only adds cost).  Guesses a quarter above
+      // it, a quarter above that, ... until one fits; then three rounds of bisection
+      // between the last two: T ends within a few percent of the least feasible one.
+      {
+        uint32_t guess = t_sum / (uint32_t)parts;
+        t_lo = guess;
+        for (int k = 0; k < 12; ++k) {
+          guess += (guess >> 2) + 1u;
+          if (guess >= t_hi) break;
+          if (fits(guess)) {
+            t_hi = guess;
+            break;
+          }
+          t_lo = guess;
+        }
+      }
+      for (int round = 0; round < 3 && t_hi - t_lo > 1; ++round) {
+        const uint32_t t_mid = t_lo + (t_hi - t_lo) / 2;
+        if (fits(t_mid)) t_hi = t_mid; else t_lo = t_mid;
+      }
+      // chunks in request order; the request that owns chunk `part` gets its units
+      int before = 0;
+#pragma unroll
+      for (int q = 0; q < kPerLane; ++q) {
+        if (q * kWave >= p.t.n_requests) break;
+        const int n_mine = un[q] > 0 ? shrink_chunks_needed(un[q], re[q], t_hi) : 0;
+        int inc = n_mine;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+          const int up = __shfl_up(inc, o, kWave);
+          if (lane >= o) inc += up;
+        }
+        const int mine_before = before + inc - n_mine;
+        if (tid < kWave && n_mine > 0 && part >= mine_before && part < mine_before + n_mine) {
+          const int64_t i = part - mine_before;
+          const int idx = lane + q * kWave;
+          s_ub[idx] = (int)((int64_t)un[q] * i / n_mine);
+          s_ue[idx] = (int)((int64_t)un[q] * (i + 1) / n_mine);
+          s_first = idx;
+          s_last = idx;
+        }
+        before += __shfl(inc, kWave - 1, kWave);
+      }
+      __syncthreads();
+    }
     // everything read back from LDS is the same in every lane: say so, so that the
     // tile code keeps it in scalar registers and branches on it uniformly
     auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
