@@ -10,6 +10,8 @@
 // Replaces slora/models/peft/triton_kernel/lora/lora_prefill.py:10-164 of the
 // reference.
 
+#include <type_traits>
+
 #include "common.hpp"
 #include "cabi_util.hpp"
 #ifdef SLORA_TIMING_PREFILL
@@ -139,14 +141,14 @@ __device__ __forceinline__ void swap_halves(u32x4& a, u32x4& b) {
   }
 }
 
-// One wavefront's share of the K loop of a 64-token x (16 * NT)-rank tile: the
-// 64-k blocks wave, wave + 8, ...  A block's fragments are loaded in line order
+// One wavefront's share of the K loop of a (16 * MF)-token x (16 * NT)-rank tile: the
+// 64-k blocks wave, wave + kShrWaves, ...  A block's fragments are loaded in line order
 // (xline / wline: the rows of the lane's two loads per fragment) and converted when
 // they are multiplied; the loads of one block are in flight while the previous one
 // is multiplied.  No load sits inside a branch (the wait counters then stay
 // exact): the main loop only runs where all of its blocks exist, and the tail
 // re-reads the last block where one does not.
-template <typename T, int NT>
+template <typename T, int NT, int MF>
 __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kShrMF][2],
                                               const uint16_t* const (&wline)[4][2], int wave, int piece, int h_in,
                                               f32x4 (&acc)[kShrMF][4]) {
@@ -155,7 +157,7 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
   if (n <= 0) return;
   const bool ragged_k = (h_in & 63) != 0;
   struct Block {
-    u32x4 a[kShrMF][2], b[NT][2];
+    u32x4 a[MF][2], b[NT][2];
   };
   auto load_block = [&](int i, Block& blk) {
     if (i >= n) i = n - 1;
@@ -163,7 +165,7 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
     const bool k_in = k < h_in;
     if (!k_in) k = 0;
 #pragma unroll
-    for (int f = 0; f < kShrMF; ++f)
+    for (int f = 0; f < MF; ++f)
 #pragma unroll
       for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16(xline[f][g] + k);
 #pragma unroll
@@ -172,14 +174,14 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
       for (int g = 0; g < 2; ++g) blk.b[t][g] = ldg16(wline[t][g] + k);
     if (ragged_k && !k_in) {
 #pragma unroll
-      for (int f = 0; f < kShrMF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();
+      for (int f = 0; f < MF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();
 #pragma unroll
       for (int t = 0; t < NT; ++t) blk.b[t][0] = blk.b[t][1] = zero16();
     }
   };
   auto mul_block = [&](Block& blk) {
 #pragma unroll
-    for (int f = 0; f < kShrMF; ++f) swap_halves(blk.a[f][0], blk.a[f][1]);
+    for (int f = 0; f < MF; ++f) swap_halves(blk.a[f][0], blk.a[f][1]);
 #pragma unroll
     for (int t = 0; t < NT; ++t) swap_halves(blk.b[t][0], blk.b[t][1]);
 #pragma unroll
@@ -187,7 +189,7 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int f = 0; f < kShrMF; ++f) acc[f][t] = mfma16<T>(blk.a[f][s], blk.b[t][s], acc[f][t]);
+        for (int f = 0; f < MF; ++f) acc[f][t] = mfma16<T>(blk.a[f][s], blk.b[t][s], acc[f][t]);
   };
   Block c0, c1;
   load_block(0, c0);
@@ -258,11 +260,21 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-      switch (n_tiles) {
-        case 1: shrink_k_loop<T, 1>(xline, wline, wave, piece, p.h_in, acc); break;
-        case 2: shrink_k_loop<T, 2>(xline, wline, wave, piece, p.h_in, acc); break;
-        case 3: shrink_k_loop<T, 3>(xline, wline, wave, piece, p.h_in, acc); break;
-        default: shrink_k_loop<T, 4>(xline, wline, wave, piece, p.h_in, acc); break;
+      // fragments that hold no row or no rank column are neither loaded nor multiplied
+      auto k_loop = [&](auto mf) {
+        constexpr int MF = decltype(mf)::value;
+        switch (n_tiles) {
+          case 1: shrink_k_loop<T, 1, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+          case 2: shrink_k_loop<T, 2, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+          case 3: shrink_k_loop<T, 3, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+          default: shrink_k_loop<T, 4, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+        }
+      };
+      switch ((m_cnt + 15) >> 4) {
+        case 1: k_loop(std::integral_constant<int, 1>{}); break;
+        case 2: k_loop(std::integral_constant<int, 2>{}); break;
+        case 3: k_loop(std::integral_constant<int, 3>{}); break;
+        default: k_loop(std::integral_constant<int, 4>{}); break;
       }
       // C tile: lane holds column lr, rows 4*lg + i
       float* mine = s_part + wave * (kShrTM * kShrLd);
