@@ -33,6 +33,8 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80683464,  # 74392008 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70349094,     # the q/k/v launch
+    ("c3", "sgmm_expand_kernel<BF16, 2>"): 280176242,  # 154150514 read + 126025728 written
+    ("c3", "sgmm_shrink_kernel<BF16>"): 142842872,     # 140873720 read + 1969152 written
 }
 
 
@@ -354,7 +356,7 @@ def main_prefill(args, torch, device):
         "config": {"workload": w.name, "layers": L, "tokens": T, "requests": int(seg.lens_np.size),
                    "launch": args.launch, "launches_per_step": 8 * L},
         "roofline": {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dom["frac"], "traffic": None,
+                     "unit": "GB/s", "frac": dom["frac"], "traffic": TRAFFIC_BYTES.get(("c3", dom["kernel"])),
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"]},
         "kernels": kernels,
     }
