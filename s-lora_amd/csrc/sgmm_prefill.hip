@@ -95,7 +95,7 @@ struct SegShrinkArgs {
 };
 
 constexpr int kShrThreads = 256;
-constexpr int kShrWaves = kShrThreads / kWave;  // K is split over the 8 wavefronts
+constexpr int kShrWaves = kShrThreads / kWave;  // K is split over the 4 wavefronts (one per SIMD: 512 registers each)
 constexpr int kShrMF = 4;                       // 16-row A fragments per tile
 constexpr int kShrTM = 16 * kShrMF;             // token rows per tile
 constexpr int kShrNB = 64;                      // rank columns per pass
@@ -304,7 +304,7 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
 // 16 token rows: the unit work is shared out in
 constexpr int kShrUnit = 16;
 constexpr int kShrMaxGrid = 256;  // one workgroup per compute unit
-constexpr int kShrChunk = 256;    // requests described at a time (keeps two workgroups' LDS within a compute unit)
+constexpr int kShrChunk = 256;    // requests described at a time (one per thread)
 
 // inclusive prefix sum of `v` over the workgroup; *total receives the sum
 __device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave, int64_t* total) {
@@ -332,7 +332,7 @@ __device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave,
 // Cost of walking `units` 16-row units of a rank-r request as tiles of up to kShrMF units, in
 // eighths of what a weight row costs: measured per tile 6.7 us + 0.2 us per weight row, plus
 // 0.177 us per activation row (hidden 4096; all three scale alike with the hidden size).
-// 32-bit: callers keep units below 2^16.
+// 32-bit: callers keep a request to 4096 units, so that 256 requests still sum below 2^32.
 constexpr uint32_t kShrCostUnit = 7 * kShrUnit;
 __device__ __forceinline__ uint32_t shrink_tile_cost(int r_eff) { return 268u + 8u * (uint32_t)r_eff; }
 __device__ __forceinline__ uint32_t shrink_chunk_cost(int units, int r_eff) {
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
   }
   // Few requests: no workgroup is given rows of two requests (each would cost it a tile's
   // fixed share); request j is cut into n_j even chunks, one workgroup each.
-  const bool aligned = p.t.n_requests <= kShrChunk && p.t.n_requests <= parts && p.m_tiles < (1 << 14);
+  const bool aligned = p.t.n_requests <= kShrChunk && p.t.n_requests <= parts && p.m_tiles <= 1024;
   int64_t carry = 0;  // cost in front of the current chunk of requests
   for (int c0 = 0; c0 < p.t.n_requests; c0 += kShrChunk) {
     int64_t base_li = 0;
@@ -597,6 +597,7 @@ struct SegExpandArgs {
   int scales_dtype;
   int feat_out, max_rank, qkvo, m_tiles, m_span, n_chunks;
   int vec_ok;
+  int row_cap;  // rows of a request at or past this are not touched (max_input_len, rounded up to a row tile)
 };
 
 constexpr int kExpThreads = 256;
@@ -609,6 +610,7 @@ constexpr int kExpGroup = kExpOB * kExpWaves;   // outputs per workgroup: 512 co
 #define SLORA_EXP_SPAN_TILES 16
 #endif
 constexpr int kExpSpanTiles = SLORA_EXP_SPAN_TILES;  // most row tiles a workgroup walks
+constexpr int kExpWalkGrid = 768;                    // workgroups of the walking kernel: three per compute unit
 constexpr int kExpMinGrid = 512;                     // shorter spans rather than fewer workgroups than this
 
 template <typename T>
@@ -898,6 +900,105 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
   expand_mfma<T, KS>(p, r, r_eff, base_li, scale, row0, m0, m_end, nb, s_delta);
 }
 
+// The same work for batches of up to kExpReqs requests, shared out evenly: every
+// workgroup of an output group gets the same number of row tiles, whatever the
+// requests' lengths, and pays the lookups of a request (adapter, start, scale) once,
+// from LDS.  Thread j describes request j (two dependent groups of loads, outside
+// every branch); a prefix sum over the requests' tile counts lays them end to end;
+// workgroup (group, slice) walks tiles [total * slice / slices, total * (slice + 1) / slices)
+// of that line, request by request.
+constexpr int kExpReqs = 256;
+
+template <typename T, int KS>
+__global__ __launch_bounds__(kExpThreads) void sgmm_expand_walk_kernel(const SegExpandArgs p) {
+  extern __shared__ __align__(16) char s_delta[];
+  __shared__ int s_row0[kExpReqs], s_rows[kExpReqs], s_rank[kExpReqs], s_tile0[kExpReqs];
+  __shared__ int64_t s_base[kExpReqs];
+  __shared__ float s_scale[kExpReqs];
+  __shared__ int s_wsum[kExpWaves];
+  __shared__ int s_first;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int group = (int)blockIdx.x % p.n_chunks;
+  const int slice = (int)blockIdx.x / p.n_chunks, slices = (int)gridDim.x / p.n_chunks;
+
+  // request tid: an invalid one re-reads entry 0 and gets no tiles
+  const bool mine = tid < p.t.n_requests;
+  const int rq = mine ? tid : 0;
+  const int64_t a = p.t.b_indicies[rq];
+  int row0 = p.t.b_start_loc[rq];
+  int rows = p.t.b_seq_len[rq];
+  const bool a_ok = (uint64_t)a < (uint64_t)p.t.n_adapters;
+  const int64_t a_safe = a_ok ? a : 0;
+  const int64_t len = p.t.a_len[a_safe];
+  const int64_t start = p.t.a_start[a_safe];
+  const float scale = load_scale(p.scales, p.scales_dtype, a_safe);
+  const int r = (int)(len >> 2);
+  const bool valid = mine && a_ok && row0 >= 0 && rows > 0 && row0 < p.t.n_tokens && r > 0 && p.max_rank > 0;
+  if (valid) {
+    if (rows > p.t.n_tokens - row0) rows = p.t.n_tokens - row0;
+    if (rows > p.row_cap) rows = p.row_cap;
+  } else {
+    rows = 0;
+  }
+  const int tiles = (rows + kExpTMW - 1) / kExpTMW;
+  int inc = tiles;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const int up = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += up;
+  }
+  if (lane == kWave - 1) s_wsum[wave] = inc;
+  if (tid == 0) s_first = 0;
+  __syncthreads();
+  int before = 0, total = 0;
+#pragma unroll
+  for (int wv = 0; wv < kExpWaves; ++wv) {
+    const int c = s_wsum[wv];
+    if (wv < wave) before += c;
+    total += c;
+  }
+  const int tile0 = before + inc - tiles;  // tiles in front of my request
+  const int t_begin = (int)((int64_t)total * slice / slices), t_end = (int)((int64_t)total * (slice + 1) / slices);
+  s_row0[tid] = row0;
+  s_rows[tid] = rows;
+  s_rank[tid] = r;
+  s_tile0[tid] = tile0;
+  s_base[tid] = start + (int64_t)r * p.qkvo;
+  s_scale[tid] = scale;
+  if (tiles > 0 && t_begin >= tile0 && t_begin < tile0 + tiles) s_first = tid;
+  __syncthreads();
+  if (t_begin >= t_end) return;
+
+  auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  const int nb = group * kExpGroup + wave * kExpOB;
+  int t = t_begin;
+  for (int j = uni(s_first); t < t_end && j < p.t.n_requests; ++j) {
+    const int rows_j = uni(s_rows[j]);
+    const int tiles_j = (rows_j + kExpTMW - 1) / kExpTMW;
+    const int tile0_j = uni(s_tile0[j]);
+    if (tiles_j == 0 || t >= tile0_j + tiles_j) continue;
+    const int last = t_end - tile0_j < tiles_j ? t_end - tile0_j : tiles_j;  // my tiles of request j: [t - tile0_j, last)
+    const int m0 = (t - tile0_j) * kExpTMW;
+    const int m_end = last * kExpTMW < rows_j ? last * kExpTMW : rows_j;
+    t = tile0_j + last;
+    const int rj = uni(s_rank[j]);
+    const int r_eff = rj < p.max_rank ? rj : p.max_rank;
+    const int rw0 = uni(s_row0[j]);
+    const int64_t bl = s_base[j];
+    const int64_t base_li =
+        (int64_t)(((uint64_t)(uint32_t)uni((int)((uint64_t)bl >> 32)) << 32) | (uint32_t)uni((int)(uint32_t)bl));
+    const float scale_j = __builtin_bit_cast(float, uni(__builtin_bit_cast(int, s_scale[j])));
+    if (!p.vec_ok || (rj & 7) != 0 || (r_eff & 7) != 0 || r_eff > 128) {
+      const int n0 = group * kExpGroup;
+      const int n_end = n0 + kExpGroup < p.feat_out ? n0 + kExpGroup : p.feat_out;
+      expand_generic<T>(p, rj, r_eff, base_li, scale_j, rw0, m0, m_end - m0, n0, n_end - n0);
+    } else {
+      expand_mfma<T, KS>(p, rj, r_eff, base_li, scale_j, rw0, m0, m_end, nb, s_delta);
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -948,16 +1049,24 @@ int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
 
 template <typename T, int KS>
 int launch_seg_expand_ks(const SegExpandArgs& p, int64_t grid, hipStream_t stream) {
-  auto kernel = sgmm_expand_kernel<T, KS>;
+  const bool walk = p.t.n_requests <= kExpReqs && p.t.n_tokens <= (1 << 22);  // tile counts stay far inside 32 bits
+  auto kernel = walk ? sgmm_expand_walk_kernel<T, KS> : sgmm_expand_kernel<T, KS>;
   constexpr int lds = 2 * kExpChunkRows * kExpLdsRow<KS>;  // 68 KiB for ranks up to 128
-  static bool attr_done = lds <= 64 * 1024;  // benign if two threads race: the call is idempotent
-  if (!attr_done) {
+  static bool attr_done[2] = {lds <= 64 * 1024, lds <= 64 * 1024};  // benign if two threads race: the call is idempotent
+  if (!attr_done[walk]) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             lds) != hipSuccess) {
       (void)hipGetLastError();
       return SLORA_ERR_LAUNCH;
     }
-    attr_done = true;
+    attr_done[walk] = true;
+  }
+  if (walk) {
+    // as many slices per output group as fill the chip, at most one per row tile
+    const int64_t tiles = ((int64_t)p.t.n_tokens + kExpTMW - 1) / kExpTMW + p.t.n_requests;
+    int64_t slices = (kExpWalkGrid + p.n_chunks - 1) / p.n_chunks;
+    if (slices > tiles) slices = tiles;
+    grid = slices * p.n_chunks;
   }
   hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kExpThreads), lds, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
@@ -1053,6 +1162,7 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
          n_requests * ((max_input_len + kExpTMW * tiles - 1) / (kExpTMW * tiles)) * p.n_chunks < kExpMinGrid)
     tiles >>= 1;
   p.m_span = (int)(kExpTMW * tiles);
+  p.row_cap = max_input_len > (1 << 30) ? (1 << 30) : (int)((max_input_len + kExpTMW - 1) / kExpTMW * kExpTMW);
   p.m_tiles = (int)((max_input_len + p.m_span - 1) / p.m_span);
   p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
              (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
