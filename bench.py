@@ -33,8 +33,8 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80683464,  # 74392008 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70349094,     # the q/k/v launch
-    ("c3", "sgmm_expand_kernel<BF16, 2>"): 280176242,  # 154150514 read + 126025728 written
-    ("c3", "sgmm_shrink_kernel<BF16>"): 142842872,     # 140873720 read + 1969152 written
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 291811050,  # 165785322 read + 126025728 written
+    ("c3", "sgmm_shrink_kernel<BF16>"): 142855054,          # 140885902 read + 1969152 written
 }
 
 
@@ -339,7 +339,7 @@ def main_prefill(args, torch, device):
     flops = seg.flops(w, H)
     for label, sweep, kname, nbytes in (
             ("shrink", shrink_sweep, "sgmm_shrink_kernel<BF16>", seg.shrink_bytes(w)),
-            ("expand", expand_sweep, "sgmm_expand_kernel<BF16, 2>", seg.expand_bytes(w, H))):
+            ("expand", expand_sweep, "sgmm_expand_walk_kernel<BF16, 2>", seg.expand_bytes(w, H))):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
         kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
                           "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
