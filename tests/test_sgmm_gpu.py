@@ -76,6 +76,30 @@ def test_prefill_many_requests(gpu, n_req, lo, hi):
         check(c, g, p, 64, gpu, seed=p)
 
 
+@pytest.mark.parametrize("lens", [
+    [1500] + [3] * 40,                 # one long request among short ones
+    [2049],                            # a single request cut into many chunks
+    [700, 1, 64, 65, 128, 129, 16, 15, 17, 32, 33],   # lengths around the unit, tile and chunk sizes
+    [5] * 256,                         # as many requests as one pass describes
+    [40] * 255 + [900],                # ... with a long one at the end
+], ids=["skewed", "single", "boundaries", "256-short", "255-and-long"])
+def test_prefill_work_split(gpu, lens):
+    """Request mixes that exercise how the kernels share out the work: per-request
+    chunks (shrink), even shares of row tiles walked across request boundaries
+    (expand), both with fewer requests than workgroups and with more."""
+    lens = np.asarray(lens, dtype=np.int32)
+    ranks = [64, 8, 32, 16]
+    rng = np.random.default_rng(int(lens.sum()))
+    ids = np.sort(rng.integers(0, len(ranks), size=len(lens))).astype(np.int64)
+    start = np.zeros(len(lens), dtype=np.int32)
+    start[1:] = np.cumsum(lens)[:-1]
+    c = make_case(77, 320, ranks, batch=int(lens.sum()), dtype="bf16", bins=np.repeat(ids, lens))
+    c.start, c.lens, c.ids = start, lens, ids
+    g = GpuCase(c, gpu)
+    for p in (1, 3):
+        check(c, g, p, 64, gpu, seed=p)
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_prefill_random_configurations(gpu, seed):
     """Seeded random shapes for the segmented kernels: hidden any multiple of 8 up
