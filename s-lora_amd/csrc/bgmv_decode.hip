@@ -254,7 +254,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 #pragma unroll
     for (int c = 0; c < kVecPerPass; ++c) {
       const int v = c * kWave + lane;
-      wv[i][c] = __builtin_nontemporal_load(src + (v < nvec ? v : 0));
+      wv[i][c] = ldg16_stream(src + (v < nvec ? v : 0));
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -546,7 +546,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
   for (int c = 0; c < kVecPerPass; ++c) {
     const int e = (c * kWave + lane) * 8;
-    wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wpage + e)) : zero16();
+    wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16_stream(wpage + e) : zero16();
   }
   u32x4 xv[kTT];
 #pragma unroll
@@ -560,7 +560,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
       for (int c = 0; c < kVecPerPass; ++c) {
         const int e = e0 + (c * kWave + lane) * 8;
-        wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wpage + e)) : zero16();
+        wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16_stream(wpage + e) : zero16();
       }
     }
     // this lane's 8 consecutive outputs of the pass
@@ -569,7 +569,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
     u32x4 yv[kTT];
 #pragma unroll
     for (int t = 0; t < kTT; ++t)
-      yv[t] = (t < it.n_tok && y_ok) ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(y + (int64_t)it.tok[t] * h_stride + n_mine)) : zero16();
+      yv[t] = (t < it.n_tok && y_ok) ? ldg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine) : zero16();
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
       if (t < it.n_tok) {
@@ -593,7 +593,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
             const uint16_t hi = T::add((uint16_t)(yv[t][q] >> 16), (uint16_t)(dv[q] >> 16));
             out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
           }
-          __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(y + (int64_t)it.tok[t] * h_stride + n_mine));
+          stg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine, out);
         }
       }
     }

@@ -67,6 +67,14 @@ __device__ __forceinline__ float load_scale(const void* scales, int scales_dtype
 
 // ---- 16-byte accesses ------------------------------------------------------
 __device__ __forceinline__ u32x4 ldg16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+// 16 bytes that this launch reads once (weight pages) or reads and writes once (outputs):
+// nontemporal, so they do not push reused lines (activations, tables) out of the caches.
+__device__ __forceinline__ u32x4 ldg16_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void stg16_stream(void* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
 __device__ __forceinline__ u32x4 zero16() { return u32x4{0u, 0u, 0u, 0u}; }
 
 // Accesses to data that another workgroup of the SAME launch produces or

@@ -720,7 +720,7 @@ __device__ __forceinline__ void expand_load_rows(const SegExpandArgs& p, int row
     for (int g = 0; g < 2; ++g) {
       const int m = m0w + f * 16 + 8 * g + (lr & 7);
       const int64_t row = row0 + (m < m_end ? m : m_safe);
-      st.y[f][g] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(og + row * p.o_stride + (n_line < p.feat_out ? n_line : 0)));
+      st.y[f][g] = ldg16_stream(og + row * p.o_stride + (n_line < p.feat_out ? n_line : 0));
     }
 }
 
@@ -811,7 +811,7 @@ __device__ __forceinline__ void expand_finish(const SegExpandArgs& p, float scal
     for (int g = 0; g < 2; ++g) {
       const int m = m0w + f * 16 + 8 * g + (lr & 7);
       if (m < m_end && n_line < p.feat_out)
-        __builtin_nontemporal_store(out[g], reinterpret_cast<u32x4*>(og + (int64_t)(row0 + m) * p.o_stride + n_line));
+        stg16_stream(og + (int64_t)(row0 + m) * p.o_stride + n_line, out[g]);
     }
   }
 }
