@@ -254,7 +254,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 #pragma unroll
     for (int c = 0; c < kVecPerPass; ++c) {
       const int v = c * kWave + lane;
-      wv[i][c] = ldg16_stream(src + (v < nvec ? v : 0));
+      wv[i][c] = COH ? src[v < nvec ? v : 0] : ldg16_stream(src + (v < nvec ? v : 0));
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -546,7 +546,8 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
   for (int c = 0; c < kVecPerPass; ++c) {
     const int e = (c * kWave + lane) * 8;
-    wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16_stream(wpage + e) : zero16();
+    const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
+    wv[c] = w_ok ? (COH ? ldg16(wpage + e) : ldg16_stream(wpage + e)) : zero16();
   }
   u32x4 xv[kTT];
 #pragma unroll
@@ -560,7 +561,8 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
       for (int c = 0; c < kVecPerPass; ++c) {
         const int e = e0 + (c * kWave + lane) * 8;
-        wv[c] = (d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end) ? ldg16_stream(wpage + e) : zero16();
+        const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
+        wv[c] = w_ok ? (COH ? ldg16(wpage + e) : ldg16_stream(wpage + e)) : zero16();
       }
     }
     // this lane's 8 consecutive outputs of the pass
@@ -568,8 +570,10 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
     const bool y_ok = lane * 8 < out_per_pass && n_mine < n_end;
     u32x4 yv[kTT];
 #pragma unroll
-    for (int t = 0; t < kTT; ++t)
-      yv[t] = (t < it.n_tok && y_ok) ? ldg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine) : zero16();
+    for (int t = 0; t < kTT; ++t) {
+      const uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
+      yv[t] = (t < it.n_tok && y_ok) ? (COH ? ldg16(yp) : ldg16_stream(yp)) : zero16();
+    }
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
       if (t < it.n_tok) {
@@ -593,7 +597,11 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
             const uint16_t hi = T::add((uint16_t)(yv[t][q] >> 16), (uint16_t)(dv[q] >> 16));
             out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
           }
-          stg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine, out);
+          uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
+          if (COH)
+            *reinterpret_cast<u32x4*>(yp) = out;
+          else
+            stg16_stream(yp, out);
         }
       }
     }
