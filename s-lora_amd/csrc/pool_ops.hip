@@ -58,12 +58,12 @@ __global__ __launch_bounds__(256) void pool_scatter_kernel(const ScatterArgs p) 
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t v = v0 + u * 256 + threadIdx.x;
-        t[u] = ldg16(s + ((v < nvec ? v : 0) << 4));
+        t[u] = ldg16_stream(s + ((v < nvec ? v : 0) << 4));
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int64_t v = v0 + u * 256 + threadIdx.x;
-        if (v < nvec) *reinterpret_cast<u32x4*>(d + (v << 4)) = t[u];
+        if (v < nvec) stg16_stream(d + (v << 4), t[u]);
       }
     }
   } else {
