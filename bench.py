@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0
 # a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
 # None where not measured.
 TRAFFIC_BYTES = {
-    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 80683464,  # 74392008 read + 6291456 written
-    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 70349094,     # the q/k/v launch
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81403867,  # 75112411 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 71000741,     # the q/k/v launch
     ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 291811050,  # 165785322 read + 126025728 written
     ("c3", "sgmm_shrink_kernel<BF16>"): 142855054,          # 140885902 read + 1969152 written
 }
