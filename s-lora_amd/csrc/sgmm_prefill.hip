@@ -606,10 +606,7 @@ constexpr int kExpMF = 2;                       // 16-row MFMA fragments per row
 constexpr int kExpTMW = 16 * kExpMF;            // token rows per row tile
 constexpr int kExpOB = 64;                      // outputs per wavefront
 constexpr int kExpGroup = kExpOB * kExpWaves;   // outputs per workgroup: 512 contiguous bytes of every row
-#ifndef SLORA_EXP_SPAN_TILES
-#define SLORA_EXP_SPAN_TILES 16
-#endif
-constexpr int kExpSpanTiles = SLORA_EXP_SPAN_TILES;  // most row tiles a workgroup walks
+constexpr int kExpSpanTiles = 16;                    // most row tiles a workgroup of the per-request kernel walks
 constexpr int kExpWalkGrid = 768;                    // workgroups of the walking kernel: three per compute unit
 constexpr int kExpMinGrid = 512;                     // shorter spans rather than fewer workgroups than this
 
