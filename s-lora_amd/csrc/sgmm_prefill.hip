@@ -565,9 +565,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
           shrink_generic<T>(p, r_eff, base_li, rw0, m0, m_end - m0);
           __syncthreads();
         } else {
-#ifndef SLORA_PROBE_SKIP_TILE
           shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li);
-#endif
 #ifdef SLORA_TIMING_PREFILL
           if (tid == 0 && p.dbg[(size_t)blockIdx.x * 4 + 2] == 0ull)
             p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
