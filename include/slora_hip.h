@@ -46,7 +46,7 @@ extern "C" {
 #define SLORA_OK 0
 #define SLORA_ERR_NULL_POINTER -1  /* a required pointer is NULL */
 #define SLORA_ERR_BAD_DTYPE -2     /* dtype is not F16/BF16 (scales: F16/BF16/F32) */
-#define SLORA_ERR_BAD_SHAPE -3     /* negative size, qkvo outside 0..3, stride too small */
+#define SLORA_ERR_BAD_SHAPE -3     /* negative size, qkvo outside 0..3, stride too small, page ids over an empty pool */
 #define SLORA_ERR_UNSUPPORTED -4   /* "No suitable kernel": width not a multiple of 8, rank above 512, ... */
 #define SLORA_ERR_ALIGNMENT -5     /* a buffer the kernels read 16 bytes at a time is not 16-byte aligned */
 #define SLORA_ERR_LAUNCH -6        /* the HIP runtime refused the launch */

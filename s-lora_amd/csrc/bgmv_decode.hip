@@ -1110,6 +1110,7 @@ int fill_tables(Tables& t, const slora_tables* in, const int64_t* bins, int64_t 
   if (in == nullptr || in->a_start == nullptr || in->a_len == nullptr || in->a_loc == nullptr || bins == nullptr)
     return SLORA_ERR_NULL_POINTER;
   if (in->n_adapters < 0 || in->n_loc < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n_pages == 0 && in->n_loc > 0) return SLORA_ERR_BAD_SHAPE;  // page ids, but no pool they could name
   t.a_start = in->a_start;
   t.a_len = in->a_len;
   t.a_loc = in->a_loc;

@@ -1003,6 +1003,7 @@ int fill_seg_tables(SegTables& t, const slora_tables* in, const int32_t* b_start
       b_start_loc == nullptr || b_seq_len == nullptr || b_indicies == nullptr)
     return SLORA_ERR_NULL_POINTER;
   if (in->n_adapters < 0 || in->n_loc < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n_pages == 0 && in->n_loc > 0) return SLORA_ERR_BAD_SHAPE;  // page ids, but no pool they could name
   if (n_requests > (1 << 24) || n_tokens > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
   t.a_start = in->a_start;
   t.a_len = in->a_len;

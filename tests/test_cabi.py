@@ -68,6 +68,7 @@ def test_shrink_argument_checks(lib):
     assert f(P, P, P, C.byref(t), P, 8, 4096, 64, 2048, 100, 0, A.DTYPE_F16, None) == A.ERR_UNSUPPORTED  # row > page
     assert f(P, P, P, C.byref(t), P, 8, 4096, 1024, 4096, 100, 0, A.DTYPE_F16, None) == A.ERR_UNSUPPORTED  # rank cap
     assert f(P, P + 2, P, C.byref(t), P, 8, 4096, 64, 4096, 100, 0, A.DTYPE_F16, None) == A.ERR_ALIGNMENT
+    assert f(P, P, P, C.byref(t), P, 8, 4096, 64, 4096, 0, 0, A.DTYPE_F16, None) == A.ERR_BAD_SHAPE      # empty pool
 
 
 def test_expand_argument_checks(lib):
@@ -92,6 +93,7 @@ def test_sgmm_argument_checks(lib):
     assert s(P, P, P, C.byref(t), P, P, P, 4, 16, 64, 4096, 64, 4000, 4096, 64, 100, 0, A.DTYPE_BF16, None) == A.ERR_BAD_SHAPE
     assert s(P, P, P, C.byref(t), None, P, P, 4, 16, 64, 4096, 64, 4096, 4096, 64, 100, 0, A.DTYPE_BF16, None) == A.ERR_NULL_POINTER
     assert s(P, P, P, C.byref(t), P, P, P, 4, 16, 64, 4096, 64, 4096, 4096, 64, 100, 0, 3, None) == A.ERR_BAD_DTYPE
+    assert s(P, P, P, C.byref(t), P, P, P, 4, 16, 64, 4096, 64, 4096, 4096, 64, 0, 0, A.DTYPE_BF16, None) == A.ERR_BAD_SHAPE
     e = lib.slora_sgmm_expand
     assert e(P, P, P, C.byref(t), P, A.DTYPE_F16, P, P, P, 0, 0, 0, 4096, 4096, 64, 64, 4096, 4096, 100, 0, A.DTYPE_F16, None) == A.OK
     assert e(P, P, P, C.byref(t), None, A.DTYPE_F16, P, P, P, 4, 16, 64, 4096, 4096, 64, 64, 4096, 4096, 100, 0, A.DTYPE_F16, None) == A.ERR_NULL_POINTER
