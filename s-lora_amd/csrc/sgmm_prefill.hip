@@ -88,6 +88,7 @@ struct SegShrinkArgs {
   SegTables t;
   int64_t x_stride, w_stride, o_stride;  // elements per row
   int h_in, max_rank, qkvo, m_tiles;
+  int col_split;  // 1, 2 or 4 workgroups share a tile's rank columns (16-column tiles t with t % col_split == group)
   int vec_ok;  // every row start is 16-byte aligned and h_in % 8 == 0
 #ifdef SLORA_TIMING_PREFILL
   unsigned long long* dbg;  // [grid][4] clock stamps: start, requests described, first tile done, end
@@ -207,11 +208,13 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
 }
 
 // One tile: token rows row_first .. row_first + m_cnt (m_cnt <= kShrTM) of a request
-// whose weight rows start at a_loc[base_li].  All threads of the workgroup call it
-// together; it ends with a barrier.
+// whose weight rows start at a_loc[base_li]; of every 64 rank columns the 16-column
+// tiles t with t % p.col_split == cg.  All threads of the workgroup call it together;
+// it ends with a barrier.
 template <typename T>
 __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_part, int64_t row_first, int m_cnt,
-                                            int r_eff, int64_t base_li) {
+                                            int r_eff, int64_t base_li, int cg) {
+  const int cs = p.col_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
@@ -234,7 +237,10 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
 
   for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
     const int nb_cnt = p.max_rank - nb0 < kShrNB ? p.max_rank - nb0 : kShrNB;
-    if (nb0 < r_eff) {
+    // this workgroup's tiles of the pass: cg, cg + cs, ...; n_own of them hold columns of the adapter
+    const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
+    const int n_own = n_tiles > cg ? (n_tiles - cg + cs - 1) / cs : 0;
+    if (n_own > 0) {
       // weight rows of the lane's two loads per B fragment: the page lookups go out
       // together; a row that does not exist (j >= r_eff, bad page id) reads pool page
       // 0 -- its products only reach output columns that are zeroed below
@@ -245,15 +251,14 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
         for (int t = 0; t < 4; ++t)
 #pragma unroll
           for (int g = 0; g < 2; ++g) {
-            const int j = nb0 + t * 16 + 8 * g + lrow;
-            pg[t][g] = seg_page_nobranch(p.t, base_li + j, j < r_eff && p.t.n_loc > 0);
+            const int j = nb0 + (cg + cs * t) * 16 + 8 * g + lrow;
+            pg[t][g] = seg_page_nobranch(p.t, base_li + j, t < n_own && j < r_eff && p.t.n_loc > 0);
           }
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
           for (int g = 0; g < 2; ++g) wline[t][g] = wg + (pg[t][g] >= 0 ? pg[t][g] : 0) * p.w_stride;
       }
-      const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
       f32x4 acc[kShrMF][4];
 #pragma unroll
       for (int f = 0; f < kShrMF; ++f)
@@ -263,7 +268,7 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
       // fragments that hold no row or no rank column are neither loaded nor multiplied
       auto k_loop = [&](auto mf) {
         constexpr int MF = decltype(mf)::value;
-        switch (n_tiles) {
+        switch (n_own) {
           case 1: shrink_k_loop<T, 1, MF>(xline, wline, wave, piece, p.h_in, acc); break;
           case 2: shrink_k_loop<T, 2, MF>(xline, wline, wave, piece, p.h_in, acc); break;
           case 3: shrink_k_loop<T, 3, MF>(xline, wline, wave, piece, p.h_in, acc); break;
@@ -276,19 +281,22 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
         case 3: k_loop(std::integral_constant<int, 3>{}); break;
         default: k_loop(std::integral_constant<int, 4>{}); break;
       }
-      // C tile: lane holds column lr, rows 4*lg + i
+      // C tile: lane holds column lr, rows 4*lg + i; fragment t is column tile cg + cs * t
       float* mine = s_part + wave * (kShrTM * kShrLd);
 #pragma unroll
       for (int f = 0; f < kShrMF; ++f)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
+          if (t < n_own) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) mine[(f * 16 + lg * 4 + i) * kShrLd + t * 16 + lr] = acc[f][t][i];
+            for (int i = 0; i < 4; ++i)
+              mine[(f * 16 + lg * 4 + i) * kShrLd + (cg + cs * t) * 16 + lr] = acc[f][t][i];
+          }
     }
     __syncthreads();
     for (int idx = tid; idx < kShrTM * kShrNB; idx += kShrThreads) {
       const int m = idx / kShrNB, c = idx - m * kShrNB;
-      if (m < m_cnt && c < nb_cnt) {
+      if (m < m_cnt && c < nb_cnt && ((c >> 4) & (cs - 1)) == cg) {
         float v = 0.f;
         if (nb0 + c < r_eff) {
 #pragma unroll
@@ -334,7 +342,7 @@ __device__ __forceinline__ int64_t shrink_block_scan(int64_t v, int64_t* s_wave,
 // 0.177 us per activation row (hidden 4096; all three scale alike with the hidden size).
 // 32-bit: callers keep a request to 4096 units, so that 256 requests still sum below 2^32.
 constexpr uint32_t kShrCostUnit = 7 * kShrUnit;
-__device__ __forceinline__ uint32_t shrink_tile_cost(int r_eff) { return 268u + 8u * (uint32_t)r_eff; }
+__device__ __forceinline__ uint32_t shrink_tile_cost(int r_own) { return 268u + 8u * (uint32_t)r_own; }
 __device__ __forceinline__ uint32_t shrink_chunk_cost(int units, int r_eff) {
   const uint32_t tiles = ((uint32_t)units + kShrMF - 1) / kShrMF;
   return tiles * shrink_tile_cost(r_eff) + (uint32_t)units * kShrCostUnit;
@@ -375,8 +383,10 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
   __shared__ int64_t s_base[kShrChunk];
   __shared__ int s_first, s_last;
   const int tid = threadIdx.x;
-  const int parts = (int)gridDim.x;
-  const int part = (int)(blockIdx.x & 7) * (parts >> 3) + (int)(blockIdx.x >> 3);
+  // XCD-major position of the workgroup; col_split neighbours share the rows of a part
+  const int slot = (int)(blockIdx.x & 7) * ((int)gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+  const int parts = (int)gridDim.x / p.col_split;
+  const int part = slot / p.col_split, cg = slot - part * p.col_split;
   const int row_cap = p.m_tiles * kShrTM;  // rows of a request past max_input_len are not touched
 #ifdef SLORA_TIMING_PREFILL
   if (tid == 0) {
@@ -475,6 +485,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
         const int idx = lane + q * kWave;
         un[q] = (s_rows[idx] + kShrUnit - 1) / kShrUnit;
         re[q] = s_rank[idx] < p.max_rank ? s_rank[idx] : p.max_rank;
+        re[q] = (re[q] + p.col_split - 1) / p.col_split;  // weight rows one workgroup of the split reads
         if (idx >= p.t.n_requests) un[q] = 0;
         const uint32_t c = un[q] > 0 ? shrink_chunk_cost(un[q], re[q]) : 0u;
         t_hi = c > t_hi ? c : t_hi;
@@ -562,10 +573,10 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
         if (m_end > rows) m_end = rows;
         if (m_end <= m0) continue;
         if (!p.vec_ok) {
-          shrink_generic<T>(p, r_eff, base_li, rw0, m0, m_end - m0);
+          if (cg == 0) shrink_generic<T>(p, r_eff, base_li, rw0, m0, m_end - m0);
           __syncthreads();
         } else {
-          shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li);
+          shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, cg);
 #ifdef SLORA_TIMING_PREFILL
           if (tid == 0 && p.dbg[(size_t)blockIdx.x * 4 + 2] == 0ull)
             p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
@@ -1032,14 +1043,34 @@ int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
     }
     attr_done = true;
   }
-  // one workgroup per tile of token rows, at most kShrMaxGrid, a multiple of 8
-  int64_t tiles = ((int64_t)p.t.n_tokens + kShrTM - 1) / kShrTM + p.t.n_requests;
-  const int64_t by_len = (int64_t)p.t.n_requests * p.m_tiles;
-  if (by_len < tiles) tiles = by_len;
-  int64_t grid = (tiles + 7) / 8 * 8;
+  // Workgroups: at most one per 16-row unit and kShrMaxGrid.  A small batch leaves most of
+  // them without rows while each of the others streams all weight rows of its tile, so the
+  // rank columns of a tile are then shared by 2 or 4 workgroups: the split with the least
+  // estimated time of the slowest workgroup (14.2 us + per tile 0.2 us per weight row it
+  // reads + 0.177 us per row; further tiles 6.7 us each).
+  int64_t units = ((int64_t)p.t.n_tokens + kShrUnit - 1) / kShrUnit + p.t.n_requests;
+  const int64_t by_len = (int64_t)p.t.n_requests * p.m_tiles * kShrMF;
+  if (by_len < units) units = by_len;
+  if (units <= 0) return SLORA_OK;
+  int cs = 1;
+  float best = 0.f;
+  for (int c = 1; c <= 4; c *= 2) {
+    if (c > 1 && p.max_rank < 16 * c) break;  // fewer 16-column tiles than workgroups to share them
+    const int64_t row_parts = kShrMaxGrid / c;
+    int64_t rows = (p.t.n_tokens + row_parts - 1) / row_parts;
+    rows = (rows + kShrUnit - 1) / kShrUnit * kShrUnit;
+    const float tiles = (float)((rows + kShrTM - 1) / kShrTM);
+    const float t = 14.2f + tiles * (0.2f * (float)p.max_rank / (float)c) + (tiles - 1.f) * 6.7f + 0.177f * (float)rows;
+    if (c == 1 || t < best) {
+      best = t;
+      cs = c;
+    }
+  }
+  SegShrinkArgs q = p;
+  q.col_split = cs;
+  int64_t grid = (units * cs + 8 * cs - 1) / (8 * cs) * (8 * cs);
   if (grid > kShrMaxGrid) grid = kShrMaxGrid;
-  if (grid <= 0) return SLORA_OK;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
