@@ -171,6 +171,33 @@ SLORA_API int slora_sgmm_shrink(void* o, const void* x, const void* w, const slo
                       int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
                       int dtype, void* stream);
 
+/* Prefill shrink with a per-step plan.  No counterpart in the reference: its Triton
+ * kernel (lora_prefill.py:57-102) looks up request and adapter in every program of every
+ * one of the 4 x n_layers shrink launches of a prefill step
+ * (lora_unordered_batch_infer.py:358-410), all with the same b_start_loc / b_seq_len /
+ * b_indicies.  slora_sgmm_plan_build computes the split of the requests over the
+ * workgroups once (it depends on the request lengths and adapter ranks only, not on
+ * layer or projection) into `plan` (device memory, slora_sgmm_plan_bytes() bytes, 16-byte
+ * aligned, owned by the caller); slora_sgmm_shrink_planned is slora_sgmm_shrink reading
+ * that split: same arguments, same results bit for bit.
+ *   *usable = 1: the plan was built.  0: this batch shape takes no plan (more than 256
+ *   requests, more requests than workgroups, or nothing to do) -- call slora_sgmm_shrink.
+ * slora_sgmm_shrink_planned returns SLORA_ERR_BAD_SHAPE for such a shape.  The sizes
+ * (n_requests, max_input_len, n_tokens, max_rank) must be those of the build call; a plan
+ * of another launch shape makes the kernel leave `o` untouched. */
+SLORA_API int64_t slora_sgmm_plan_bytes(void);
+SLORA_API int slora_sgmm_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables,
+                          const int32_t* b_start_loc, const int32_t* b_seq_len,
+                          const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
+                          int64_t n_tokens, int64_t max_rank, int* usable, void* stream);
+SLORA_API int slora_sgmm_shrink_planned(const void* plan, void* o, const void* x, const void* w,
+                              const slora_tables* tables, const int32_t* b_start_loc,
+                              const int32_t* b_seq_len, const int64_t* b_indicies,
+                              int64_t n_requests, int64_t max_input_len, int64_t n_tokens,
+                              int64_t h_in, int64_t max_rank, int64_t x_row_stride,
+                              int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages,
+                              int qkvo, int dtype, void* stream);
+
 /* Prefill (segmented) expand.  Replaces lora_get_qkvo_fwd_expand + _expand_fwd_kernel
  * (lora_prefill.py:105-136, 10-54).
  *   o[row, n] = T( f32(o[row, n]) + (sum_{d < r_a} f32(x[row, d]) * f32(Bt[n*r_a + d])) * f32(scales[a]) )

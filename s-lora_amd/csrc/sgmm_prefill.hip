@@ -593,6 +593,117 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
 }
 
 // ---------------------------------------------------------------------------
+// shrink with a plan: the split of the requests over the workgroups depends only on
+// the batch (request lengths, adapters' ranks), not on the layer or projection, so it
+// can be computed once per prefill step and read back by the 4 x n_layers shrink
+// calls of that step with one scalar load per workgroup.
+// ---------------------------------------------------------------------------
+constexpr int kSegPlanMagic = 0x53475031;
+constexpr int kSegPlanHeaderWords = 16;
+constexpr int kSegPartWords = 8;
+enum SegPlanHeader { SP_MAGIC = 0, SP_PARTS, SP_SPLIT, SP_NREQ, SP_NTOKENS, SP_MAXRANK, SP_ROWCAP };
+enum SegPart { PT_ROW = 0, PT_ROWS, PT_RANK, PT_START_LO, PT_START_HI };
+
+// One workgroup.  Same scheme as the few-requests case of sgmm_shrink_kernel (request j
+// in n_j even chunks, T bisected), with more rounds; record `part` = chunk `part` in
+// request order, empty records behind the last chunk.
+__global__ __launch_bounds__(kShrThreads) void sgmm_plan_kernel(int* plan, SegTables t, int parts, int col_split,
+                                                                int max_rank, int row_cap) {
+  __shared__ int64_t s_wave[kShrWaves];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < parts * kSegPartWords; i += kShrThreads) plan[kSegPlanHeaderWords + i] = 0;
+  const bool mine = tid < t.n_requests;
+  const int rq = mine ? tid : 0;
+  const int64_t a = t.b_indicies[rq];
+  const int row0 = t.b_start_loc[rq];
+  int rows = t.b_seq_len[rq];
+  const bool a_ok = (uint64_t)a < (uint64_t)t.n_adapters;
+  const int64_t len = t.a_len[a_ok ? a : 0];
+  const int64_t start = t.a_start[a_ok ? a : 0];
+  const int r = (int)(len >> 2);
+  int units = 0;
+  if (mine && a_ok && row0 >= 0 && rows > 0 && row0 < t.n_tokens) {
+    if (rows > t.n_tokens - row0) rows = t.n_tokens - row0;
+    if (rows > row_cap) rows = row_cap;
+    units = (rows + kShrUnit - 1) / kShrUnit;
+  }
+  int r_own = r < max_rank ? r : max_rank;
+  r_own = (r_own + col_split - 1) / col_split;
+  const uint32_t cost = units > 0 ? shrink_chunk_cost(units, r_own) : 0u;
+  int64_t t_sum = 0;
+  shrink_block_scan((int64_t)cost, s_wave, &t_sum);
+  // the dearest single request bounds T from above (one chunk per request always fits)
+  uint32_t t_hi = cost;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)t_hi, o, kWave);
+    t_hi = other > t_hi ? other : t_hi;
+  }
+  if ((tid & 63) == 0) s_wave[tid >> 6] = t_hi;
+  __syncthreads();
+#pragma unroll
+  for (int wv = 0; wv < kShrWaves; ++wv) t_hi = (uint32_t)s_wave[wv] > t_hi ? (uint32_t)s_wave[wv] : t_hi;
+  __syncthreads();
+  uint32_t t_lo = (uint32_t)(t_sum / parts);  // the even share: a lower bound
+  if (t_lo > t_hi) t_lo = t_hi;
+  for (int round = 0; round < 20 && t_hi - t_lo > 1; ++round) {
+    const uint32_t t_mid = t_lo + (t_hi - t_lo) / 2;
+    int64_t sum = 0;
+    shrink_block_scan(units > 0 ? shrink_chunks_needed(units, r_own, t_mid) : 0, s_wave, &sum);
+    if (sum <= parts) t_hi = t_mid; else t_lo = t_mid;
+  }
+  const int n_mine = units > 0 ? shrink_chunks_needed(units, r_own, t_hi) : 0;
+  int64_t n_all = 0;
+  const int64_t before = shrink_block_scan(n_mine, s_wave, &n_all) - n_mine;
+  for (int i = 0; i < n_mine && before + i < parts; ++i) {
+    const int ub = (int)((int64_t)units * i / n_mine), ue = (int)((int64_t)units * (i + 1) / n_mine);
+    const int m0 = ub * kShrUnit;
+    const int m_end = ue * kShrUnit < rows ? ue * kShrUnit : rows;
+    int* rec = plan + kSegPlanHeaderWords + (before + i) * kSegPartWords;
+    rec[PT_ROW] = row0 + m0;
+    rec[PT_ROWS] = m_end - m0;
+    rec[PT_RANK] = r;
+    rec[PT_START_LO] = (int)(uint32_t)start;
+    rec[PT_START_HI] = (int)((uint64_t)start >> 32);
+  }
+  if (tid == 0) {
+    plan[SP_MAGIC] = kSegPlanMagic;
+    plan[SP_PARTS] = parts;
+    plan[SP_SPLIT] = col_split;
+    plan[SP_NREQ] = t.n_requests;
+    plan[SP_NTOKENS] = t.n_tokens;
+    plan[SP_MAXRANK] = max_rank;
+    plan[SP_ROWCAP] = row_cap;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(const SegShrinkArgs p, const int* plan) {
+  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
+  const int slot = (int)(blockIdx.x & 7) * ((int)gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+  const int parts = (int)gridDim.x / p.col_split;
+  const int part = slot / p.col_split, cg = slot - part * p.col_split;
+  // header and record of this part in one group of scalar loads
+  const int* rec = plan + kSegPlanHeaderWords + part * kSegPartWords;
+  int magic = plan[SP_MAGIC], n_parts = plan[SP_PARTS], split = plan[SP_SPLIT];
+  int row_first = rec[PT_ROW], m_rows = rec[PT_ROWS], r = rec[PT_RANK], lo = rec[PT_START_LO], hi = rec[PT_START_HI];
+  asm volatile("" : "+s"(magic), "+s"(n_parts), "+s"(split), "+s"(row_first), "+s"(m_rows), "+s"(r), "+s"(lo), "+s"(hi));
+  if (magic != kSegPlanMagic || n_parts != parts || split != p.col_split) return;  // not a plan of this launch shape
+  if (m_rows <= 0 || row_first < 0 || m_rows > p.t.n_tokens - row_first) return;
+  const int r_eff = r < p.max_rank ? r : p.max_rank;
+  const int64_t base_li = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo) + (int64_t)r * p.qkvo;
+  for (int m0 = 0; m0 < m_rows; m0 += kShrTM) {
+    const int m_cnt = m_rows - m0 < kShrTM ? m_rows - m0 : kShrTM;
+    if (!p.vec_ok) {
+      if (cg == 0) shrink_generic<T>(p, r_eff, base_li, row_first, m0, m_cnt);
+      __syncthreads();
+    } else {
+      shrink_tile<T>(p, s_part, (int64_t)row_first + m0, m_cnt, r_eff, base_li, cg);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // expand
 // ---------------------------------------------------------------------------
 struct SegExpandArgs {
@@ -1030,47 +1141,63 @@ int fill_seg_tables(SegTables& t, const slora_tables* in, const int32_t* b_start
   return SLORA_OK;
 }
 
-template <typename T>
-int launch_seg_shrink(const SegShrinkArgs& p, hipStream_t stream) {
-  const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
-  auto kernel = sgmm_shrink_kernel<T>;
-  static bool attr_done = false;  // benign if two threads race: the call is idempotent
-  if (!attr_done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds) != hipSuccess) {
-      (void)hipGetLastError();
-      return SLORA_ERR_LAUNCH;
-    }
-    attr_done = true;
-  }
-  // Workgroups: at most one per 16-row unit and kShrMaxGrid.  A small batch leaves most of
-  // them without rows while each of the others streams all weight rows of its tile, so the
-  // rank columns of a tile are then shared by 2 or 4 workgroups: the split with the least
-  // estimated time of the slowest workgroup (14.2 us + per tile 0.2 us per weight row it
-  // reads + 0.177 us per row; further tiles 6.7 us each).
-  int64_t units = ((int64_t)p.t.n_tokens + kShrUnit - 1) / kShrUnit + p.t.n_requests;
-  const int64_t by_len = (int64_t)p.t.n_requests * p.m_tiles * kShrMF;
+// Workgroups of a shrink launch and how many of them share a tile's rank columns: at most
+// one workgroup per 16-row unit and kShrMaxGrid.  A small batch leaves most of them without
+// rows while each of the others streams all weight rows of its tile, so the rank columns of
+// a tile are then shared by 2 or 4 workgroups: the split with the least estimated time of
+// the slowest workgroup (14.2 us + per tile 0.2 us per weight row it reads + 0.177 us per
+// row; further tiles 6.7 us each).  grid = 0: nothing to do.
+void shrink_geometry(int64_t n_tokens, int64_t n_requests, int64_t m_tiles, int64_t max_rank, int64_t& grid, int& cs) {
+  grid = 0;
+  cs = 1;
+  int64_t units = (n_tokens + kShrUnit - 1) / kShrUnit + n_requests;
+  const int64_t by_len = n_requests * m_tiles * kShrMF;
   if (by_len < units) units = by_len;
-  if (units <= 0) return SLORA_OK;
-  int cs = 1;
+  if (units <= 0) return;
   float best = 0.f;
   for (int c = 1; c <= 4; c *= 2) {
-    if (c > 1 && p.max_rank < 16 * c) break;  // fewer 16-column tiles than workgroups to share them
+    if (c > 1 && max_rank < 16 * c) break;  // fewer 16-column tiles than workgroups to share them
     const int64_t row_parts = kShrMaxGrid / c;
-    int64_t rows = (p.t.n_tokens + row_parts - 1) / row_parts;
+    int64_t rows = (n_tokens + row_parts - 1) / row_parts;
     rows = (rows + kShrUnit - 1) / kShrUnit * kShrUnit;
     const float tiles = (float)((rows + kShrTM - 1) / kShrTM);
-    const float t = 14.2f + tiles * (0.2f * (float)p.max_rank / (float)c) + (tiles - 1.f) * 6.7f + 0.177f * (float)rows;
+    const float t = 14.2f + tiles * (0.2f * (float)max_rank / (float)c) + (tiles - 1.f) * 6.7f + 0.177f * (float)rows;
     if (c == 1 || t < best) {
       best = t;
       cs = c;
     }
   }
-  SegShrinkArgs q = p;
-  q.col_split = cs;
-  int64_t grid = (units * cs + 8 * cs - 1) / (8 * cs) * (8 * cs);
+  grid = (units * cs + 8 * cs - 1) / (8 * cs) * (8 * cs);
   if (grid > kShrMaxGrid) grid = kShrMaxGrid;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
+}
+
+// a plan holds one record per row part: usable where no part spans two requests
+bool shrink_plan_usable(int64_t n_requests, int64_t m_tiles, int64_t grid, int cs) {
+  return grid > 0 && n_requests <= kShrChunk && n_requests <= grid / cs && m_tiles <= 1024;
+}
+
+template <typename T>
+int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t stream) {
+  const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
+  int64_t grid = 0;
+  SegShrinkArgs q = p;
+  shrink_geometry(p.t.n_tokens, p.t.n_requests, p.m_tiles, p.max_rank, grid, q.col_split);
+  if (grid <= 0) return SLORA_OK;
+  if (plan != nullptr && !shrink_plan_usable(p.t.n_requests, p.m_tiles, grid, q.col_split)) return SLORA_ERR_BAD_SHAPE;
+  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T>)
+                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T>);
+  static bool attr_done[2] = {false, false};  // benign if two threads race: the call is idempotent
+  if (!attr_done[plan != nullptr]) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
+      (void)hipGetLastError();
+      return SLORA_ERR_LAUNCH;
+    }
+    attr_done[plan != nullptr] = true;
+  }
+  if (plan != nullptr)
+    hipLaunchKernelGGL(sgmm_shrink_planned_kernel<T>, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q, plan);
+  else
+    hipLaunchKernelGGL(sgmm_shrink_kernel<T>, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -1109,16 +1236,11 @@ int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
   return launch_seg_expand_ks<T, 4>(p, grid, stream);
 }
 
-}  // namespace
-}  // namespace slora
-
-extern "C" {
-
-int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables* tables, const int32_t* b_start_loc,
-                      const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
-                      int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride,
-                      int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype, void* stream) {
-  using namespace slora;
+int seg_shrink_common(const int* plan, bool planned, void* o, const void* x, const void* w, const slora_tables* tables,
+                      const int32_t* b_start_loc, const int32_t* b_seq_len, const int64_t* b_indicies,
+                      int64_t n_requests, int64_t max_input_len, int64_t n_tokens, int64_t h_in, int64_t max_rank,
+                      int64_t x_row_stride, int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
+                      int dtype, void* stream) {
   if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
   if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || h_in < 0 || max_rank < 0) return SLORA_ERR_BAD_SHAPE;
   if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
@@ -1130,6 +1252,8 @@ int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables*
   if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
   if (o == nullptr || x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
   if (h_in == 0 || h_in > (1 << 21) || max_rank > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
+  if (planned && (reinterpret_cast<uintptr_t>(plan) & 15) != 0) return SLORA_ERR_ALIGNMENT;
+  if (max_input_len > n_tokens) max_input_len = n_tokens;  // no request is longer than the batch
   p.o = o;
   p.x = x;
   p.w = w;
@@ -1140,12 +1264,71 @@ int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables*
   p.max_rank = (int)max_rank;
   p.qkvo = qkvo;
   p.m_tiles = (int)((max_input_len + kShrTM - 1) / kShrTM);
+  p.col_split = 1;
   p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
 #ifdef SLORA_TIMING_PREFILL
   p.dbg = reinterpret_cast<unsigned long long*>(strtoull(getenv("SLORA_TIMING_BUF"), nullptr, 0));
 #endif
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, s) : launch_seg_shrink<BF16>(p, s);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, plan, s) : launch_seg_shrink<BF16>(p, plan, s);
+}
+
+}  // namespace
+}  // namespace slora
+
+extern "C" {
+
+int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables* tables, const int32_t* b_start_loc,
+                      const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
+                      int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride,
+                      int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype, void* stream) {
+  return slora::seg_shrink_common(nullptr, false, o, x, w, tables, b_start_loc, b_seq_len, b_indicies, n_requests,
+                                  max_input_len, n_tokens, h_in, max_rank, x_row_stride, w_row_stride, o_row_stride,
+                                  n_pages, qkvo, dtype, stream);
+}
+
+int64_t slora_sgmm_plan_bytes(void) {
+  return (int64_t)sizeof(int) * (slora::kSegPlanHeaderWords + slora::kShrMaxGrid * slora::kSegPartWords);
+}
+
+int slora_sgmm_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables, const int32_t* b_start_loc,
+                          const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests,
+                          int64_t max_input_len, int64_t n_tokens, int64_t max_rank, int* usable, void* stream) {
+  using namespace slora;
+  if (usable == nullptr) return SLORA_ERR_NULL_POINTER;
+  *usable = 0;
+  if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || max_rank < 0) return SLORA_ERR_BAD_SHAPE;
+  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (plan_bytes < slora_sgmm_plan_bytes()) return SLORA_ERR_BAD_SHAPE;
+  if ((reinterpret_cast<uintptr_t>(plan) & 15) != 0) return SLORA_ERR_ALIGNMENT;
+  if (max_rank > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
+  if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0) return SLORA_OK;
+  SegTables t{};
+  int rc = fill_seg_tables(t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, 1);
+  if (rc != SLORA_OK) return rc;
+  if (t.n_adapters == 0) return SLORA_OK;
+  if (max_input_len > n_tokens) max_input_len = n_tokens;
+  const int64_t m_tiles = (max_input_len + kShrTM - 1) / kShrTM;
+  int64_t grid = 0;
+  int cs = 1;
+  shrink_geometry(n_tokens, n_requests, m_tiles, max_rank, grid, cs);
+  if (!shrink_plan_usable(n_requests, m_tiles, grid, cs)) return SLORA_OK;
+  hipLaunchKernelGGL(sgmm_plan_kernel, dim3(1), dim3(kShrThreads), 0, reinterpret_cast<hipStream_t>(stream),
+                     static_cast<int*>(plan), t, (int)(grid / cs), cs, (int)max_rank, (int)(m_tiles * kShrTM));
+  if (hipGetLastError() != hipSuccess) return SLORA_ERR_LAUNCH;
+  *usable = 1;
+  return SLORA_OK;
+}
+
+int slora_sgmm_shrink_planned(const void* plan, void* o, const void* x, const void* w, const slora_tables* tables,
+                              const int32_t* b_start_loc, const int32_t* b_seq_len, const int64_t* b_indicies,
+                              int64_t n_requests, int64_t max_input_len, int64_t n_tokens, int64_t h_in,
+                              int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride, int64_t o_row_stride,
+                              int64_t n_pages, int qkvo, int dtype, void* stream) {
+  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
+  return slora::seg_shrink_common(static_cast<const int*>(plan), true, o, x, w, tables, b_start_loc, b_seq_len,
+                                  b_indicies, n_requests, max_input_len, n_tokens, h_in, max_rank, x_row_stride,
+                                  w_row_stride, o_row_stride, n_pages, qkvo, dtype, stream);
 }
 
 int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables* tables, const void* scales,
@@ -1164,6 +1347,7 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
   if (page_elems == 0) page_elems = feat_out;  // the reference's convention: page width == output width
   if (x_row_stride < max_rank || w_row_stride < page_elems || o_row_stride < feat_out) return SLORA_ERR_BAD_SHAPE;
   if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0 || feat_out == 0) return SLORA_OK;
+  if (max_input_len > n_tokens) max_input_len = n_tokens;  // no request is longer than the batch
   SegExpandArgs p{};
   int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
   if (rc != SLORA_OK) return rc;

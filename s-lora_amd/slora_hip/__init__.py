@@ -10,4 +10,5 @@ from ._cabi import lib_path, load_library, version  # noqa: F401
 from ._kernels import (BgmvPlan, clear_plan_cache, dispatch_bgmv, dispatch_bgmv_lora,  # noqa: F401
                        dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_lora, dispatch_bgmv_qkv_shrink, make_plan,
                        plan_wait_timed_out, rebuild_plan)
-from .lora_prefill import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand  # noqa: F401
+from .lora_prefill import (SgmmPlan, clear_prefill_plan_cache, lora_get_qkvo_fwd_expand,  # noqa: F401
+                           lora_get_qkvo_fwd_shrink, make_prefill_plan)

@@ -45,6 +45,10 @@ SIGNATURES = {
                                        _I64, _I64, _I64, _I64, _I64, _I, _I, _P]),
     "slora_sgmm_shrink": (_I, [_P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I, _I, _P]),
+    "slora_sgmm_plan_bytes": (_I64, []),
+    "slora_sgmm_plan_build": (_I, [_P, _I64, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, C.POINTER(C.c_int), _P]),
+    "slora_sgmm_shrink_planned": (_I, [_P, _P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                       _I64, _I, _I, _P]),
     "slora_sgmm_expand": (_I, [_P, _P, _P, _TP, _P, _I, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I64, _I64, _I, _I, _P]),
     "slora_bgmv_lora_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64,

@@ -11,6 +11,18 @@ from test_bgmv_gpu import GpuCase, dev, host, RTOL, ATOL, TDT
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["cache", "no-plan"])
+def prefill_plan_mode(request, monkeypatch):
+    """Every test runs twice: with shrink calls served by the automatic per-batch plan
+    (the default) and with the cache off, which sends them to the kernel that works out
+    its share of the batch by itself."""
+    import slora_hip
+    monkeypatch.setenv("SLORA_PLAN_CACHE", "1" if request.param == "cache" else "0")
+    slora_hip.clear_prefill_plan_cache()
+    yield request.param
+    slora_hip.clear_prefill_plan_cache()
+
+
 def seg_case(seed, hidden, ranks, n_req, lo, hi, dtype, h_out=None, sort=True):
     start, lens, ids = make_segments(seed, n_req, lo, hi, len(ranks), sort_by_adapter=sort)
     T = int(lens.sum())
@@ -249,3 +261,84 @@ def test_prefill_matches_decode_kernels(gpu):
     dispatch_bgmv(y, delta, g.value, g.a_start, g.a_len, g.a_loc, g.bins, 0, g.scales)
     np.testing.assert_allclose(host(delta), d_gpu, rtol=RTOL, atol=ATOL)
     np.testing.assert_allclose(host(y), y_gpu, rtol=2 * RTOL, atol=4 * ATOL)
+
+
+def _shrink_args(c, g, device):
+    start = dev(c.start, torch.int32, device)
+    lens = dev(c.lens, torch.int32, device)
+    ids = dev(c.ids, torch.int64, device)
+    return start, lens, ids, int(c.lens.max())
+
+
+@pytest.mark.parametrize("hidden,ranks,n_req,lo,hi", [
+    (256, [8, 16, 32, 64], 9, 1, 70),       # small batch: rank columns shared by 4 workgroups
+    (1024, [64, 8, 16], 40, 30, 200),       # one chunk or a few per request
+    (320, [128, 24], 5, 1, 300),            # two passes over the rank, odd rank (element-wise path)
+    (256, [16, 32], 300, 1, 9),             # more requests than a plan describes: the plain kernel runs
+])
+def test_prefill_plan_gives_the_plain_kernels_bits(gpu, hidden, ranks, n_req, lo, hi):
+    """An explicit plan, the automatic one and no plan at all: identical outputs."""
+    from slora_hip import lora_get_qkvo_fwd_shrink, make_prefill_plan
+    c = seg_case(900 + n_req, hidden, ranks, n_req, lo, hi, "bf16")
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    R = (max(ranks) + 7) // 8 * 8
+    plan = make_prefill_plan(g.a_start, g.a_len, start, lens, ids, c.batch, R, max_len)
+    assert plan.usable == (n_req <= 256)
+    w_a = g.key.view(c.n_pages, c.page_elems)
+    for p in range(4):
+        outs = []
+        for how in (False, plan, None):
+            o = torch.full((c.batch, R), 7.0, dtype=g.tdt, device=gpu)
+            lora_get_qkvo_fwd_shrink(g.x, w_a, o, g.a_loc, g.a_start, g.a_len, start, lens, ids, c.hidden, p, R,
+                                     max_len, plan=how)
+            outs.append(o)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), p
+
+
+def test_prefill_plan_cache_follows_the_index_tensors(gpu, prefill_plan_mode):
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_prefill
+    if prefill_plan_mode != "cache":
+        pytest.skip("cache switched off")
+    c = seg_case(31, 256, [16, 8, 32], 12, 1, 90, "f16")
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    w_a = g.key.view(c.n_pages, c.page_elems)
+    cache = lora_prefill._prefill_plan_cache
+    cache.hits = cache.builds = 0
+
+    def both(lens_t, ids_t):
+        o0 = torch.full((c.batch, 32), 3.0, dtype=g.tdt, device=gpu)  # rows of no request keep this value
+        o1 = o0.clone()
+        lora_get_qkvo_fwd_shrink(g.x, w_a, o0, g.a_loc, g.a_start, g.a_len, start, lens_t, ids_t, c.hidden, 2, 32,
+                                 max_len, plan=False)
+        lora_get_qkvo_fwd_shrink(g.x, w_a, o1, g.a_loc, g.a_start, g.a_len, start, lens_t, ids_t, c.hidden, 2, 32,
+                                 max_len)
+        torch.cuda.synchronize()
+        assert torch.equal(o0, o1)
+
+    both(lens, ids)
+    both(lens, ids)
+    assert (cache.builds, cache.hits) == (1, 1)
+    ids.copy_(torch.flip(ids, dims=[0]))          # in place: the version changes, the plan is rebuilt
+    both(lens, ids)
+    assert cache.builds == 2
+    lens2 = lens.clone()                          # another object with the same values: rebuilt as well
+    both(lens2, ids)
+    assert cache.builds == 3
+    lens2[0] = 0                                  # a request dropped in place
+    both(lens2, ids)
+    assert cache.builds == 4
+
+
+def test_prefill_plan_of_another_batch_is_rejected(gpu):
+    from slora_hip import lora_get_qkvo_fwd_shrink, make_prefill_plan
+    c = seg_case(32, 256, [16, 8], 6, 1, 50, "f16")
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    plan = make_prefill_plan(g.a_start, g.a_len, start, lens, ids, c.batch, 16, max_len)
+    o = torch.zeros((c.batch, 32), dtype=g.tdt, device=gpu)
+    with pytest.raises(RuntimeError, match="another batch"):
+        lora_get_qkvo_fwd_shrink(g.x, g.key.view(c.n_pages, c.page_elems), o, g.a_loc, g.a_start, g.a_len, start, lens,
+                                 ids, c.hidden, 0, 32, max_len, plan=plan)
