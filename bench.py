@@ -34,7 +34,7 @@ TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81403867,  # 75112411 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 71000741,     # the q/k/v launch
     ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 291811050,  # 165785322 read + 126025728 written
-    ("c3", "sgmm_shrink_kernel<BF16>"): 142855054,          # 140885902 read + 1969152 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16>"): 142855054,  # 140885902 read + 1969152 written
 }
 
 
@@ -313,10 +313,16 @@ def main_prefill(args, torch, device):
     d = torch.zeros((T, R), device=device, dtype=w.dtype)
     t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
 
+    def plan():  # once per prefill step, as the automatic cache does for a caller that passes none
+        return slora_hip.make_prefill_plan(w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies, T, R,
+                                           seg.max_len)
+
     def shrink_sweep():
+        pl = plan()
         for l in range(L):
             for p in range(4):
-                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len)
+                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len,
+                                                   plan=pl)
 
     def expand_sweep():
         for l in range(L):
@@ -325,9 +331,11 @@ def main_prefill(args, torch, device):
                                                    seg.max_len)
 
     def step():
+        pl = plan()
         for l in range(L):
             for p in range(4):
-                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len)
+                slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len,
+                                                   plan=pl)
                 slora_hip.lora_get_qkvo_fwd_expand(d, w.value_buffer[l].view(-1, H), y[l], w.a_scaling, *t, H, p, R,
                                                    seg.max_len)
 
@@ -338,7 +346,7 @@ def main_prefill(args, torch, device):
     kernels = {}
     flops = seg.flops(w, H)
     for label, sweep, kname, nbytes in (
-            ("shrink", shrink_sweep, "sgmm_shrink_kernel<BF16>", seg.shrink_bytes(w)),
+            ("shrink", shrink_sweep, "sgmm_shrink_planned_kernel<BF16>", seg.shrink_bytes(w)),
             ("expand", expand_sweep, "sgmm_expand_walk_kernel<BF16, 2>", seg.expand_bytes(w, H))):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
         kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
@@ -354,7 +362,7 @@ def main_prefill(args, torch, device):
         "n_gpus": 1, "steps": reps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w.name, "layers": L, "tokens": T, "requests": int(seg.lens_np.size),
-                   "launch": args.launch, "launches_per_step": 8 * L},
+                   "launch": args.launch, "launches_per_step": 8 * L + 1},
         "roofline": {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": dom["frac"], "traffic": TRAFFIC_BYTES.get(("c3", dom["kernel"])),
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"]},
