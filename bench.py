@@ -33,8 +33,8 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81403867,  # 75112411 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 71000741,     # the q/k/v launch
-    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 291811050,  # 165785322 read + 126025728 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16>"): 142855054,  # 140885902 read + 1969152 written
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281674768,  # 155648888 read + 126025879 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16>"): 142878462,  # 140909310 read + 1969152 written
 }
 
 
