@@ -112,23 +112,38 @@ class _PrefillPlanCache:
     for the very same tensor objects (weak references) at the same ``_version``, sizes and
     stream; nothing is cached during graph capture; ``SLORA_PLAN_CACHE=0`` turns it off."""
 
+    MISS_STREAK = 8   # builds in a row that no later call reused ...
+    COOL_DOWN = 256   # ... switch the cache off for this many calls: the caller makes new tensors every time
+
     def __init__(self, capacity: int = 2):
         self.capacity = capacity
         self.entries = []
         self.hits = 0
         self.builds = 0
+        self.streak = 0
+        self.paused = 0
 
     def clear(self) -> None:
         self.entries.clear()
+        self.streak = self.paused = 0
 
     def get(self, tensors, sizes, stream):
+        if self.paused:
+            self.paused -= 1
+            return None
         versions = tuple(t._version for t in tensors)
         for i, (refs, vers, sz, strm, plan) in enumerate(self.entries):
             if sz == sizes and strm == stream and vers == versions and all(r() is t for r, t in zip(refs, tensors)):
                 if i:
                     self.entries.insert(0, self.entries.pop(i))
                 self.hits += 1
+                self.streak = 0
                 return plan
+        self.streak += 1
+        if self.streak > self.MISS_STREAK:
+            self.streak = 0
+            self.paused = self.COOL_DOWN
+            return None
         plan = make_prefill_plan(*tensors, *sizes)
         self.builds += 1
         self.entries.insert(0, (tuple(weakref.ref(t) for t in tensors), versions, sizes, stream, plan))

@@ -330,6 +330,10 @@ def test_prefill_plan_cache_follows_the_index_tensors(gpu, prefill_plan_mode):
     lens2[0] = 0                                  # a request dropped in place
     both(lens2, ids)
     assert cache.builds == 4
+    # a caller that makes new tensors for every call gets no plan after a few useless builds
+    for _ in range(cache.MISS_STREAK + 3):
+        both(lens2.clone(), ids)
+    assert cache.paused > 0 and cache.builds <= 4 + cache.MISS_STREAK
 
 
 def test_prefill_plan_of_another_batch_is_rejected(gpu):
