@@ -727,7 +727,9 @@ constexpr int kExpTMW = 16 * kExpMF;            // token rows per row tile
 constexpr int kExpOB = 64;                      // outputs per wavefront
 constexpr int kExpGroup = kExpOB * kExpWaves;   // outputs per workgroup: 512 contiguous bytes of every row
 constexpr int kExpSpanTiles = 16;                    // most row tiles a workgroup of the per-request kernel walks
-constexpr int kExpWalkGrid = 768;                    // workgroups of the walking kernel: three per compute unit
+// workgroups of the walking kernel: as many per compute unit as its registers allow (156; 224 for ranks above 64)
+template <int KS>
+constexpr int kExpWalkGrid = KS <= 2 ? 768 : 512;
 constexpr int kExpMinGrid = 512;                     // shorter spans rather than fewer workgroups than this
 
 template <typename T>
@@ -1218,7 +1220,7 @@ int launch_seg_expand_ks(const SegExpandArgs& p, int64_t grid, hipStream_t strea
   if (walk) {
     // as many slices per output group as fill the chip, at most one per row tile
     const int64_t tiles = ((int64_t)p.t.n_tokens + kExpTMW - 1) / kExpTMW + p.t.n_requests;
-    int64_t slices = (kExpWalkGrid + p.n_chunks - 1) / p.n_chunks;
+    int64_t slices = (kExpWalkGrid<KS> + p.n_chunks - 1) / p.n_chunks;
     if (slices > tiles) slices = tiles;
     grid = slices * p.n_chunks;
   }
