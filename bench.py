@@ -20,7 +20,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "s-lora_amd")):
+for _p in (ROOT, os.path.join(ROOT, "s-lora_amd"), os.path.join(ROOT, "tests")):  # tests/: the workload builder
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -49,12 +49,11 @@ def parse_args():
                     help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels; "
                          "load: copying adapters into the pool; the last two are reported in the same format with "
                          "their own metric names")
-    ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused", "planned-lora"],
+    ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused"],
                     default="planned-fused",
                     help="dropin: 8 stateless dispatch_bgmv calls per layer exactly as the reference issues them; "
                          "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer); "
-                         "planned*: the same with a per-step plan (built inside every timed step) passed as plan=; "
-                         "planned-lora: shrink and expand of q/k/v in one launch and of o in another (2 per layer)")
+                         "planned*: the same with a per-step plan (built inside every timed step) passed as plan=")
     ap.add_argument("--all-modes", action="store_true", help="also time the other modes and report them under 'modes'")
     ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
                     help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
@@ -99,7 +98,6 @@ def make_step(w, bufs, mode):
     t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
     planned = mode.startswith("planned")
     fused = mode.endswith("fused")
-    lora = mode.endswith("lora")
     plan = slora_hip.make_plan(*t, w.max_rank, w.n_pages) if planned else None
     kw = {"plan": plan} if planned else {}
     L = w.n_layers
@@ -113,15 +111,6 @@ def make_step(w, bufs, mode):
     def qkv_expand(l):
         slora_hip.dispatch_bgmv_qkv_expand(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
                                            bufs.delta[2], w.value_buffer[l], *t, w.a_scaling, **kw)
-
-    def qkv_lora(l):
-        slora_hip.dispatch_bgmv_qkv_lora(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
-                                         bufs.delta[2], bufs.x_in[l], w.key_buffer[l], w.value_buffer[l], *t,
-                                         w.a_scaling, **kw)
-
-    def o_lora(l):
-        slora_hip.dispatch_bgmv_lora(bufs.y[l][3], bufs.delta[0], bufs.x_att[l], w.key_buffer[l], w.value_buffer[l],
-                                     *t, 3, w.a_scaling, **kw)
 
     def shrink(l, p):
         bgmv(bufs.delta[p % 3], bufs.x_in[l] if p < 3 else bufs.x_att[l], w.key_buffer[l], *t, p, w.a_scaling, **kw)
@@ -143,14 +132,7 @@ def make_step(w, bufs, mode):
         return sweep
 
     sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
-    if lora:
-        families = {
-            "qkv_lora": (over_layers(qkv_lora), f"bgmv_lora_kernel<{ty}, 3>", L,
-                         w.qkv_shrink_bytes() + w.qkv_expand_bytes()),
-            "o_lora": (over_layers(o_lora), f"bgmv_lora_kernel<{ty}, 1>", L,
-                       w.shrink_bytes() + w.expand_bytes(w.h_out[3])),
-        }
-    elif fused:
+    if fused:
         families = {
             "qkv_shrink": (over_layers(qkv_shrink), sk, L, w.qkv_shrink_bytes()),
             "o_shrink": (over_layers(shrink, 3), sk, L, w.shrink_bytes()),
@@ -170,10 +152,6 @@ def make_step(w, bufs, mode):
             # a new batch every step: calls that pass no plan may reuse one only within the step
             slora_hip.clear_plan_cache()
         for l in range(L):
-            if lora:
-                qkv_lora(l)
-                o_lora(l)
-                continue
             if fused:
                 qkv_shrink(l)
                 qkv_expand(l)
@@ -302,7 +280,7 @@ MFMA_PEAK_TFLOPS = 2500.0
 def main_prefill(args, torch, device):
     """C3: q/k/v/o segmented shrink and expand over a prefill batch, per layer."""
     import slora_hip
-    from slora_hip import workloads
+    import workloads
     L = min(args.layers, 4)
     w, seg = workloads.c3_prefill(device, n_layers=L)
     T, H, R = seg.n_tokens, w.hidden, w.max_rank
@@ -478,7 +456,7 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     import slora_hip
-    from slora_hip import workloads
+    import workloads
     slora_hip.load_library()
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
@@ -503,7 +481,7 @@ def main():
         w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024)
     bufs = StepBuffers(w, device)
     step, families = make_step(w, bufs, args.mode)
-    fused = args.mode.endswith("fused") or args.mode.endswith("lora")
+    fused = args.mode.endswith("fused")
     if args.check:
         check_layer0(w, bufs, torch)
 
@@ -529,15 +507,14 @@ def main():
     ms_per_step = time_steps(run_step)
     other_modes = {}
     if args.all_modes:
-        for m in ("dropin", "fused", "planned", "planned-fused", "planned-lora"):
+        for m in ("dropin", "fused", "planned", "planned-fused"):
             if m == args.mode:
                 continue
             st, _ = make_step(w, bufs, m)
             fn = graphed(st, torch) if use_graph else st
             ms = time_steps(fn)
             other_modes[m] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1),
-                              "launches_per_step": w.n_layers * (2 if m.endswith("lora") else
-                                                                 4 if m.endswith("fused") else 8)}
+                              "launches_per_step": w.n_layers * (4 if m.endswith("fused") else 8)}
 
     # ---- launch duration of every kind of launch in the step: a sweep of that kind over
     # all layers, HIP events on the stream the kernels run on (back-to-back launches, so
@@ -575,7 +552,7 @@ def main():
             "pool_pages_per_layer": w.n_pages,
             "mode": args.mode,
             "launch": args.launch,
-            "launches_per_step": w.n_layers * (2 if args.mode.endswith("lora") else 4 if fused else 8) +
+            "launches_per_step": w.n_layers * (4 if fused else 8) +
                                  (1 if args.mode.startswith("planned") else 0),
         },
         "step_hbm": {

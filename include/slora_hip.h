@@ -212,25 +212,6 @@ SLORA_API int slora_sgmm_expand(void* o, const void* x, const void* w, const slo
                       int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
                       int dtype, void* stream);
 
-/* Shrink and expand of the same projections in ONE launch: what the reference does
- * with two back-to-back dispatch_bgmv calls per projection
- * (slora/models/peft/lora_unordered_batch_infer.py:267-273, 287-295, 307-315,
- * 428-448).  delta_p = shrink(x) through the A pool w_a exactly as
- * slora_bgmv_shrink_planned writes it, then y_p += expand(delta_p) through the B
- * pool w_b exactly as slora_bgmv_expand_planned: same results bit for bit, one
- * kernel boundary less per pair.  nproj = 3 takes q, k, v (qkvo must be 0), nproj
- * = 1 the projection qkvo.  Inside the launch the expand workgroups wait on
- * per-run counters kept behind the plan's items (hence a non-const plan); a plan
- * must not be used by two such launches at the same time (two streams).  The
- * counters are left at zero.  Hidden sizes above 16384 are not supported here
- * (SLORA_ERR_UNSUPPORTED): issue the two calls. */
-SLORA_API int slora_bgmv_lora_planned(void* plan, int64_t rank_cap, int64_t n_items, int nproj, void* delta0,
-                            void* delta1, void* delta2, void* y0, void* y1, void* y2, const void* x,
-                            const void* w_a, const void* w_b, const slora_tables* tables, const int64_t* bins,
-                            const void* scales, int scales_dtype, int64_t batch, int64_t h_in, int64_t delta_cols,
-                            int64_t h_out0, int64_t h_out1, int64_t h_out2, int64_t page_elems, int64_t n_pages,
-                            int qkvo, int dtype, void* stream);
-
 /* ---- moving adapters in and out of the pool --------------------------------- */
 
 /* pool[loc[i]] = rows[i], i < n_rows, for n_bufs pool buffers in one go.

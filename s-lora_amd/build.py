@@ -23,7 +23,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-fvisibility=hidden",
     "-Wall",
     "-Wno-unused-function",
@@ -39,10 +38,7 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found; libslora_hip.so cannot be built")
 
 
-def build_library(verbose: bool = True) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC, *srcs, "-o", LIB_PATH]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -51,6 +47,23 @@ def build_library(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
     if verbose and out.strip():
         print(out, flush=True)
+
+
+def build_library(verbose: bool = True) -> str:
+    """Compile every source to an object (in parallel, one hipcc each), then link."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(HERE, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = hipcc_path()
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", CSRC]
+    jobs = []
+    for s in SOURCES:
+        obj = os.path.join(obj_dir, os.path.splitext(s)[0] + ".o")
+        jobs.append((obj, [hipcc, *HIPCC_FLAGS, *inc, "-c", os.path.join(CSRC, s), "-o", obj]))
+    with ThreadPoolExecutor(max_workers=min(len(jobs), 8)) as pool:
+        list(pool.map(lambda j: _run(j[1], verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[j[0] for j in jobs], "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 

@@ -61,13 +61,6 @@ __device__ __forceinline__ int64_t lookup_page(const Tables& t, int64_t li) {
 //   [42]     1 if this is the run's last stored item and rank > rank_cap (rows the plan does not list)
 constexpr int kPlanMagic = 0x534c5032;  // "SLP2"
 constexpr int kPlanHeaderWords = 16;
-// Counters behind a plan's items and scratch, for launches that hold both shrink
-// and expand: [SY_TIMEOUT] set if a wavefront ever gave up waiting, then two
-// counters per (token, projection), used at the first token of a run: shrink
-// workgroups of the run that are done, expand wavefronts of the run that are done.
-// They only grow (by at most 8 * rank / 8 per launch) until the plan is rebuilt.
-constexpr int kSyncHeader = 4;
-enum { SY_TIMEOUT = 1 };
 constexpr int kItemWords = 48;
 enum { PH_MAGIC = 0, PH_NITEMS = 1, PH_MAXRANK = 2, PH_BATCH = 3, PH_TT = 4, PH_RANKCAP = 5, PH_NRUNS = 6 };
 enum { IT_ADAPTER = 0, IT_RANK = 1, IT_NTOK = 2, IT_J0 = 3, IT_TOK = 4, IT_PAGES = 8, IT_BASE = 40, IT_MORE = 42 };
@@ -226,7 +219,7 @@ struct ShrinkArgs {
 // load is unconditional (absent tokens / rows read a valid dummy address and are
 // discarded) so that no branch separates the loads: first the activations, then
 // both weight pages; the LDS stores wait for the activations only.
-template <typename T, bool COH>
+template <typename T>
 __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it, int proj, int r_eff,
                                             const int64_t (&page)[2], u32x4* s_x) {
   const int tid = threadIdx.x, lane = tid & 63;
@@ -254,7 +247,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 #pragma unroll
     for (int c = 0; c < kVecPerPass; ++c) {
       const int v = c * kWave + lane;
-      wv[i][c] = COH ? src[v < nvec ? v : 0] : ldg16_stream(src + (v < nvec ? v : 0));
+      wv[i][c] = ldg16_stream(src + (v < nvec ? v : 0));
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -295,11 +288,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
       if (t < it.n_tok) {
         const float sum = wave_sum(acc[i][t]);
         if (lane == 0 && page[i] >= 0 && row < r_eff) {
-          uint16_t* dst = y + (int64_t)it.tok[t] * p.y_cols + row;
-          if (COH)
-            st16_coherent(dst, T::from_float(sum));
-          else
-            *dst = T::from_float(sum);
+          y[(int64_t)it.tok[t] * p.y_cols + row] = T::from_float(sum);
         }
       }
     }
@@ -310,12 +299,9 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 // q/k/v call launches three workgroups per item (projection-major, so that with
 // a multiple of 8 items all three run on the item's XCD and share its
 // activations in that L2).
-// `block` = projection * units + item.  s_x: [lds_tt][h_in / 8] LDS words.  `key`
-// receives first token * 4 + projection of the item's run (-1: no run), which names
-// the run's completion counter when shrink and expand share one launch.
-// COH: the rows are read by expand workgroups of the same launch (see common.hpp).
-template <typename T, bool PLANNED, bool COH>
-__device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x4* s_x, int& key) {
+// `block` = projection * units + item.  s_x: [lds_tt][h_in / 8] LDS words.
+template <typename T, bool PLANNED>
+__device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x4* s_x) {
   constexpr int NW = 4;
   constexpr int NTASK = 2;
   constexpr int NT = NW * kWave;
@@ -335,7 +321,6 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
     discover_run(p.t, p.batch, b, it);
     it.j0 = (unit - b * p.blocks) * kRB;
   }
-  key = it.n_tok > 0 ? it.tok[0] * 4 + p.qkvo0 + proj : -1;
   // page ids of this wavefront's two rows, read before any branch
   int64_t page2[2];
 #pragma unroll
@@ -356,7 +341,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       if (it.j0 + wave + 4 * i >= r_eff) page2[i] = -1;
-    shrink_fast<T, COH>(p, it, proj, r_eff, page2, s_x);
+    shrink_fast<T>(p, it, proj, r_eff, page2, s_x);
     return;
   }
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
@@ -462,11 +447,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
           if (t < nt) {
             const float s = wave_sum(acc[i][t]);
             if (lane == 0 && wrow[i] != nullptr) {
-              uint16_t* dst = y + (int64_t)item_token(it, t0 + t) * p.y_cols + row[i];
-              if (COH)
-                st16_coherent(dst, T::from_float(s));
-              else
-                *dst = T::from_float(s);
+              y[(int64_t)item_token(it, t0 + t) * p.y_cols + row[i]] = T::from_float(s);
             }
           }
         }
@@ -478,8 +459,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
 template <typename T, bool PLANNED>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];  // [lds_tt][h_in / 8]
-  int key;
-  shrink_body<T, PLANNED, false>(p, (int)blockIdx.x, s_x, key);
+  shrink_body<T, PLANNED>(p, (int)blockIdx.x, s_x);
 }
 
 // ---------------------------------------------------------------------------
@@ -496,9 +476,6 @@ struct ExpandArgs {
   int scales_dtype;
   int batch, x_cols, qkvo0, blocks, y_aligned, units;
   int h_out[3];
-  int* sync;       // shared launch of shrink and expand only: the plan's counters
-  int rank_cap;    //   the plan's rank_cap
-  int spin_limit;  //   polls after which a waiting wavefront gives up
 };
 
 // Reduce the 8 partial sums of a pass over the LPO lanes that share an output
@@ -522,7 +499,7 @@ __device__ __forceinline__ void file_sums(const float (&part)[kVecPerPass], floa
 // scaled sums of a pass are transposed through a 1 KiB LDS strip of the
 // wavefront so that the read-modify-write of y is one 16-byte load and one
 // 16-byte store per lane and token.
-template <typename T, bool COH>
+template <typename T>
 __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const Item& it, int r_eff,
                                             const uint16_t* wpage, int64_t flat0, float scale, uint16_t* s_strip) {
   const int lane = threadIdx.x & 63;
@@ -547,14 +524,12 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
   for (int c = 0; c < kVecPerPass; ++c) {
     const int e = (c * kWave + lane) * 8;
     const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
-    wv[c] = w_ok ? (COH ? ldg16(wpage + e) : ldg16_stream(wpage + e)) : zero16();
+    wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
   }
   u32x4 xv[kTT];
 #pragma unroll
   for (int t = 0; t < kTT; ++t)
-    xv[t] = !(t < it.n_tok && d_ok) ? zero16()
-            : COH                   ? ldg16_coherent(x + (int64_t)it.tok[t] * p.x_cols + d0)
-                                    : ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0);
+    xv[t] = (t < it.n_tok && d_ok) ? ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0) : zero16();
 
   for (int e0 = 0; e0 < page_elems; e0 += kPassElems) {
     if (e0 != 0) {
@@ -562,7 +537,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
       for (int c = 0; c < kVecPerPass; ++c) {
         const int e = e0 + (c * kWave + lane) * 8;
         const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
-        wv[c] = w_ok ? (COH ? ldg16(wpage + e) : ldg16_stream(wpage + e)) : zero16();
+        wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
       }
     }
     // this lane's 8 consecutive outputs of the pass
@@ -572,7 +547,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
       const uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
-      yv[t] = (t < it.n_tok && y_ok) ? (COH ? ldg16(yp) : ldg16_stream(yp)) : zero16();
+      yv[t] = (t < it.n_tok && y_ok) ? ldg16_stream(yp) : zero16();
     }
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
@@ -597,11 +572,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
             const uint16_t hi = T::add((uint16_t)(yv[t][q] >> 16), (uint16_t)(dv[q] >> 16));
             out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
           }
-          uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
-          if (COH)
-            *reinterpret_cast<u32x4*>(yp) = out;
-          else
-            stg16_stream(yp, out);
+          stg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine, out);
         }
       }
     }
@@ -611,7 +582,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 // Any rank, any alignment: one lane per output whose first element lies in this
 // page, element-wise loads through a_loc (an output's r elements may continue
 // on the next page).
-template <typename T, bool COH>
+template <typename T>
 __device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, const Item& it, int r_eff, int k,
                                               int64_t base_li, float scale) {
   const int h_out = p.h_out[proj];
@@ -633,8 +604,7 @@ __device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, con
         const int64_t page = lookup_page(p.t, base_li + pg);
         if (page < 0) continue;
         const float wf = T::to_float(wbase[page * pe + off]);
-        const uint16_t* xp = x + (int64_t)bt * p.x_cols + d;
-        acc = __builtin_fmaf(wf, T::to_float(COH ? ld16_coherent(xp) : *xp), acc);
+        acc = __builtin_fmaf(wf, T::to_float(x[(int64_t)bt * p.x_cols + d]), acc);
       }
       uint16_t* yp = y + (int64_t)bt * h_out + n;
       *yp = T::add(*yp, T::from_float(acc * scale));
@@ -644,29 +614,27 @@ __device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, con
 
 // Page kk of projection `proj` for the item's run; `page` is its pool page id
 // or -2 to look it up in a_loc.
-template <typename T, bool COH>
+template <typename T>
 __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const Item& it, int r_eff, int kk,
                                            int64_t page, bool vec_ok, uint16_t* s_strip) {
   const int64_t base_li = it.base + (int64_t)it.r * (p.qkvo0 + proj);
   if (!vec_ok) {
-    expand_scalar<T, COH>(p, proj, it, r_eff, kk, base_li, load_scale(p.scales, p.scales_dtype, it.a));
+    expand_scalar<T>(p, proj, it, r_eff, kk, base_li, load_scale(p.scales, p.scales_dtype, it.a));
     return;
   }
   if (page == -2) page = lookup_page(p.t, base_li + kk);
   if (page < 0) return;
   const uint16_t* wpage = reinterpret_cast<const uint16_t*>(p.w) + page * p.page_elems;
   const int64_t flat0 = (int64_t)kk * p.page_elems;
-  expand_page<T, COH>(p, proj, it, r_eff, wpage, flat0, load_scale(p.scales, p.scales_dtype, it.a), s_strip);
+  expand_page<T>(p, proj, it, r_eff, wpage, flat0, load_scale(p.scales, p.scales_dtype, it.a), s_strip);
 }
 
 // Expand has nothing to share between wavefronts (the delta row is 16 bytes per
 // lane), so every wavefront takes exactly one page: a workgroup is 4 wavefronts
 // = half of one projection's 8-page block of an item, and an item gets
 // 2 * NPROJ workgroups.
-// `block` = (projection * 2 + half) * units + item.  With FUSED the launch also holds
-// the shrink workgroups that produce x: a wavefront that has something to do first
-// waits until all of them for its run and projection have counted themselves in.
-template <typename T, int NPROJ, bool PLANNED, bool FUSED>
+// `block` = (projection * 2 + half) * units + item.
+template <typename T, int NPROJ, bool PLANNED>
 __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint16_t* s_strip) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   // sub-block major: with a multiple of 8 units, every workgroup of a unit lands on XCD unit % 8
@@ -701,45 +669,19 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint
   else
     extra = it.j0 + kRB >= p.blocks * kRB;
   const bool has_work = k < n_pg || extra;
-  if (!FUSED && !has_work) return;
+  if (!has_work) return;
   const bool pow2 = (r & (r - 1)) == 0;
   // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
   const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
                       (p.page_elems % (8 * r)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
-  // FUSED: two counters per (first token of the run, projection), never reset while
-  // the plan lives: cnt[0] counts shrink workgroups of the run that have stored
-  // their rows (`need` per launch), cnt[1] expand wavefronts of the run that are
-  // through (8 per item, with or without work: 8 * need per launch).  Between
-  // launches both are whole multiples; during launch n cnt[1] stays below
-  // (n + 1) * 8 * need as long as this wavefront has not checked out itself, so its
-  // value tells n, and the rows are complete once cnt[0] reaches (n + 1) * need.
-  const int listed = r < p.rank_cap ? r : p.rank_cap;
-  const int need = (listed + kRB - 1) / kRB;  // the run's items = its shrink workgroups per projection
-  int* cnt = FUSED ? p.sync + kSyncHeader + (it.tok[0] * 4 + p.qkvo0 + proj) * 2 : nullptr;
-  if (FUSED && has_work) {
-    const int out = __hip_atomic_load(cnt + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const int target = (out / (2 * 4 * need) + 1) * need;
-    int spins = 0;
-    while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-      if (++spins > p.spin_limit) {  // never expected; leaves a mark instead of waiting for ever
-        p.sync[SY_TIMEOUT] = 1;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(16);
-    }
-    // the rows are read with device-scope loads (ldg16_coherent); keep them behind the poll
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  }
   if (k < n_pg) {
     const int64_t page = PLANNED ? (int64_t)plan_pg : (int64_t)-2;
-    expand_one<T, FUSED>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
+    expand_one<T>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
   }
   if (extra) {
 #pragma unroll 1
-    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T, FUSED>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
+    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
   }
-  if (FUSED && (threadIdx.x & 63) == 0)  // check out; nobody waits for the result
-    __hip_atomic_fetch_add(cnt + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------
@@ -783,8 +725,7 @@ enum { SC_ADAPTER = 0, SC_TOKEN = 1, SC_RANK = 2, SC_ITEMS = 3, SC_WORK = 4, SC_
 // single L2.  Queues are padded to the longest with empty items.
 __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict__ plan, Tables t, int batch,
                                                                  int rank_cap, int max_items,
-                                                                 int* __restrict__ scratch, int* __restrict__ sync) {
-  for (int i = threadIdx.x; i < kSyncHeader + 8 * batch; i += kPlanThreads) sync[i] = 0;
+                                                                 int* __restrict__ scratch) {
   __shared__ int s_bins[kMaxLdsBins];
   __shared__ int s_ra[kMaxLdsRuns], s_rb[kMaxLdsRuns], s_rn[kMaxLdsRuns];
   __shared__ int s_wave[kPlanWaves];
@@ -946,10 +887,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
 constexpr int kFastPlanBatch = 1024;
 
 __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_fast_kernel(int* __restrict__ plan, Tables t, int batch,
-                                                                      int rank_cap, int max_items,
-                                                                      int* __restrict__ sync) {
-  if (blockIdx.x == 0)
-    for (int i = threadIdx.x; i < kSyncHeader + 8 * batch; i += kPlanThreads) sync[i] = 0;
+                                                                      int rank_cap, int max_items) {
   __shared__ int s_bins[kFastPlanBatch];    // adapter of a token, -1: none
   __shared__ int s_run[kFastPlanBatch];     // token -> run, valid at a run's first token
   __shared__ int s_ra[kFastPlanBatch], s_rr[kFastPlanBatch], s_rn[kFastPlanBatch];  // run: adapter, rank, items
@@ -1131,9 +1069,7 @@ int64_t plan_max_items(int64_t batch, int64_t rank_cap) {
 }
 // int32 words of the builder's scratch area behind the items
 int64_t plan_scratch_words(int64_t batch) { return batch * SC_WORDS; }
-// int32 words of the counters behind the scratch area, and where they start
-int64_t plan_sync_words(int64_t batch) { return kSyncHeader + 8 * batch; }
-int64_t plan_sync_offset(int64_t batch, int64_t rank_cap) {
+int64_t plan_words(int64_t batch, int64_t rank_cap) {
   return kPlanHeaderWords + plan_max_items(batch, rank_cap) * kItemWords + plan_scratch_words(batch);
 }
 
@@ -1165,43 +1101,7 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
 template <typename T, int NPROJ, bool PLANNED>
 __global__ __launch_bounds__(256, 5) void bgmv_expand_kernel(const ExpandArgs p) {
   __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
-  expand_body<T, NPROJ, PLANNED, false>(p, (int)blockIdx.x, s_out[threadIdx.x >> 6]);
-}
-
-// Shrink and expand of the same projections in one launch: the first n_shrink
-// workgroups are the shrink grid, the rest the expand grid.  Workgroups are handed
-// out in index order, so every shrink workgroup is running or done before the
-// first expand workgroup starts and a waiting expand wavefront cannot starve the
-// producers it waits for.  A shrink workgroup counts itself in on its run's
-// counter after its rows are stored; an expand wavefront polls that counter before
-// it reads them, and checks out on a second counter when it is done (see
-// expand_body).  No atomic returns a value anybody waits for, and there is no
-// counter that every workgroup touches: thousands of device-scope atomics on one
-// address cost more than the launch boundary they replace.
-struct LoraArgs {
-  ShrinkArgs s;
-  ExpandArgs e;
-  int n_shrink;
-};
-
-template <typename T, int NPROJ>
-__global__ __launch_bounds__(256, 4) void bgmv_lora_kernel(const LoraArgs p) {
-  extern __shared__ u32x4 s_x[];  // shrink staging, [lds_tt][h_in / 8]
-  __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
-  int key = -1;
-  if ((int)blockIdx.x < p.n_shrink)
-    shrink_body<T, true, true>(p.s, (int)blockIdx.x, s_x, key);
-  else
-    expand_body<T, NPROJ, true, true>(p.e, (int)blockIdx.x - p.n_shrink, s_out[threadIdx.x >> 6]);
-  if ((int)blockIdx.x < p.n_shrink && key >= 0) {
-    // the rows were stored with device-scope stores (st16_coherent): once every wavefront
-    // has waited for its stores (the release fence) and reached the barrier, the
-    // workgroup counts itself in on its run's counter
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    if (threadIdx.x == 0)
-      __hip_atomic_fetch_add(p.e.sync + kSyncHeader + key * 2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  expand_body<T, NPROJ, PLANNED>(p, (int)blockIdx.x, s_out[threadIdx.x >> 6]);
 }
 
 template <typename T, int NPROJ, bool PLANNED>
@@ -1349,28 +1249,6 @@ int expand_common(const void* plan, int64_t n_items, int64_t rank_cap, void* con
                                   : dispatch_expand<BF16>(p, nproj, planned, grid, s);
 }
 
-// shrink + expand of the same projections in one launch (needs a plan)
-template <typename T>
-int launch_lora(LoraArgs p, int nproj, int64_t items, hipStream_t stream) {
-  const size_t row_bytes = (size_t)p.s.h_in * 2;
-  int tt = kTT;
-  while (tt > 1 && tt * row_bytes > 32 * 1024) --tt;
-  const size_t lds = tt * row_bytes;
-  if (lds > kLdsSoftLimit) return SLORA_ERR_UNSUPPORTED;  // hidden sizes above 16384 take the two separate launches
-  p.s.lds_tt = tt;
-  p.s.units = (int)items;
-  p.e.units = (int)items;
-  const int64_t n_shrink = items * nproj, grid = n_shrink + items * 2 * nproj;
-  if (grid <= 0) return SLORA_OK;
-  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  p.n_shrink = (int)n_shrink;
-  if (nproj == 3)
-    hipLaunchKernelGGL((bgmv_lora_kernel<T, 3>), dim3((uint32_t)grid), dim3(256), lds, stream, p);
-  else
-    hipLaunchKernelGGL((bgmv_lora_kernel<T, 1>), dim3((uint32_t)grid), dim3(256), lds, stream, p);
-  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
-}
-
 }  // namespace
 }  // namespace slora
 
@@ -1417,7 +1295,7 @@ int slora_bgmv_expand_qkv(void* y_q, void* y_k, void* y_v, const void* x_q, cons
 
 int64_t slora_bgmv_plan_bytes(int64_t batch, int64_t rank_cap) {
   if (batch < 0 || rank_cap <= 0 || rank_cap > SLORA_MAX_RANK || batch > (1 << 24)) return SLORA_ERR_BAD_SHAPE;
-  return 4 * (slora::plan_sync_offset(batch, rank_cap) + slora::plan_sync_words(batch));
+  return 4 * slora::plan_words(batch, rank_cap);
 }
 
 int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables, const int64_t* bins,
@@ -1438,13 +1316,12 @@ int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* ta
     grid = grid < 1 ? 1 : (grid > 16 ? 16 : grid);
     hipLaunchKernelGGL(bgmv_plan_fast_kernel, dim3((uint32_t)grid), dim3(kPlanThreads), 0,
                        reinterpret_cast<hipStream_t>(stream), static_cast<int*>(plan), t, (int)batch, (int)rank_cap,
-                       (int)max_items, static_cast<int*>(plan) + plan_sync_offset(batch, rank_cap));
+                       (int)max_items);
     return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
   }
   int* scratch = static_cast<int*>(plan) + kPlanHeaderWords + max_items * kItemWords;
   hipLaunchKernelGGL(bgmv_plan_kernel, dim3(1), dim3(kPlanThreads), 0, reinterpret_cast<hipStream_t>(stream),
-                     static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items, scratch,
-                     static_cast<int*>(plan) + plan_sync_offset(batch, rank_cap));
+                     static_cast<int*>(plan), t, (int)batch, (int)rank_cap, (int)max_items, scratch);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -1475,41 +1352,6 @@ int slora_bgmv_expand_planned(const void* plan, int64_t rank_cap, int64_t n_item
   const int64_t hs[3] = {h_out0, h_out1, h_out2};
   return slora::expand_common(plan, n_items, rank_cap, ys, xs, hs, nproj, qkvo, w, tables, bins, scales,
                               scales_dtype, batch, x_cols, page_elems, n_pages, dtype, stream);
-}
-
-int slora_bgmv_lora_planned(void* plan, int64_t rank_cap, int64_t n_items, int nproj, void* delta0, void* delta1,
-                            void* delta2, void* y0, void* y1, void* y2, const void* x, const void* w_a,
-                            const void* w_b, const slora_tables* tables, const int64_t* bins, const void* scales,
-                            int scales_dtype, int64_t batch, int64_t h_in, int64_t delta_cols, int64_t h_out0,
-                            int64_t h_out1, int64_t h_out2, int64_t page_elems, int64_t n_pages, int qkvo, int dtype,
-                            void* stream) {
-  using namespace slora;
-  if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
-  if (rank_cap <= 0 || rank_cap > SLORA_MAX_RANK) return SLORA_ERR_BAD_SHAPE;
-  if (nproj != 1 && nproj != 3) return SLORA_ERR_BAD_SHAPE;
-  if (nproj == 3 && qkvo != 0) return SLORA_ERR_BAD_SHAPE;
-  void* ds[3] = {delta0, delta1, delta2};
-  void* ys[3] = {y0, y1, y2};
-  const void* xs[3] = {delta0, delta1, delta2};
-  const int64_t hs[3] = {h_out0, nproj == 3 ? h_out1 : 0, nproj == 3 ? h_out2 : 0};
-  LoraArgs p{};
-  int64_t grid_s = 0, grid_e = 0;
-  int rc = shrink_prepare(plan, n_items, rank_cap, ds, nproj, qkvo, x, w_a, tables, bins, batch, h_in, delta_cols,
-                          page_elems, n_pages, dtype, p.s, grid_s);
-  if (rc != SLORA_OK) return rc == kNothingToDo ? SLORA_OK : rc;
-  rc = expand_prepare(plan, n_items, rank_cap, ys, xs, hs, nproj, qkvo, w_b, tables, bins, scales, scales_dtype,
-                      batch, delta_cols, page_elems, n_pages, dtype, p.e, grid_e);
-  if (rc == kNothingToDo) {  // no output column anywhere: the shrink alone
-    hipStream_t s0 = reinterpret_cast<hipStream_t>(stream);
-    return dtype == SLORA_DTYPE_F16 ? dispatch_shrink<F16>(p.s, nproj, true, grid_s, s0)
-                                    : dispatch_shrink<BF16>(p.s, nproj, true, grid_s, s0);
-  }
-  if (rc != SLORA_OK) return rc;
-  p.e.sync = static_cast<int*>(plan) + plan_sync_offset(batch, rank_cap);
-  p.e.rank_cap = (int)rank_cap;
-  p.e.spin_limit = 1 << 20;
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_lora<F16>(p, nproj, grid_s, s) : launch_lora<BF16>(p, nproj, grid_s, s);
 }
 
 }  // extern "C"

@@ -14,9 +14,6 @@
 
 #include "common.hpp"
 #include "cabi_util.hpp"
-#ifdef SLORA_TIMING_PREFILL
-#include <stdlib.h>
-#endif
 
 namespace slora {
 namespace {
@@ -90,9 +87,6 @@ struct SegShrinkArgs {
   int h_in, max_rank, qkvo, m_tiles;
   int col_split;  // 1, 2 or 4 workgroups share a tile's rank columns (16-column tiles t with t % col_split == group)
   int vec_ok;  // every row start is 16-byte aligned and h_in % 8 == 0
-#ifdef SLORA_TIMING_PREFILL
-  unsigned long long* dbg;  // [grid][4] clock stamps: start, requests described, first tile done, end
-#endif
 };
 
 constexpr int kShrThreads = 256;
@@ -388,12 +382,6 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
   const int parts = (int)gridDim.x / p.col_split;
   const int part = slot / p.col_split, cg = slot - part * p.col_split;
   const int row_cap = p.m_tiles * kShrTM;  // rows of a request past max_input_len are not touched
-#ifdef SLORA_TIMING_PREFILL
-  if (tid == 0) {
-    p.dbg[(size_t)blockIdx.x * 4 + 0] = __builtin_amdgcn_s_memrealtime();
-    p.dbg[(size_t)blockIdx.x * 4 + 2] = 0ull;
-  }
-#endif
 
   // request -> cost of one of its units (0: nothing to do).  The loads sit outside
   // every branch, in two dependent groups: (adapter id, first row, row count), then
@@ -556,9 +544,6 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
     // tile code keeps it in scalar registers and branches on it uniformly
     auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
     const int first = uni(s_first), last = uni(s_last);
-#ifdef SLORA_TIMING_PREFILL
-    if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 1] = __builtin_amdgcn_s_memrealtime();
-#endif
     for (int j = first; j <= last; ++j) {
       const int u0 = uni(s_ub[j]), u1 = uni(s_ue[j]);
       const int rj = uni(s_rank[j]);
@@ -577,19 +562,12 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
           __syncthreads();
         } else {
           shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, cg);
-#ifdef SLORA_TIMING_PREFILL
-          if (tid == 0 && p.dbg[(size_t)blockIdx.x * 4 + 2] == 0ull)
-            p.dbg[(size_t)blockIdx.x * 4 + 2] = __builtin_amdgcn_s_memrealtime();
-#endif
         }
       }
     }
     carry += tot;
     __syncthreads();  // the tables are rewritten by the next chunk
   }
-#ifdef SLORA_TIMING_PREFILL
-  if (tid == 0) p.dbg[(size_t)blockIdx.x * 4 + 3] = __builtin_amdgcn_s_memrealtime();
-#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -1268,9 +1246,6 @@ int seg_shrink_common(const int* plan, bool planned, void* o, const void* x, con
   p.m_tiles = (int)((max_input_len + kShrTM - 1) / kShrTM);
   p.col_split = 1;
   p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
-#ifdef SLORA_TIMING_PREFILL
-  p.dbg = reinterpret_cast<unsigned long long*>(strtoull(getenv("SLORA_TIMING_BUF"), nullptr, 0));
-#endif
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, plan, s) : launch_seg_shrink<BF16>(p, plan, s);
 }

@@ -340,96 +340,3 @@ def dispatch_bgmv_qkv_expand(y_q, y_k, y_v, x_q, x_k, x_v, w, start_indicies, lo
     if rc == _cabi.ERR_UNSUPPORTED:
         raise RuntimeError(no_kernel)
     _cabi.check(rc, "dispatch_bgmv_qkv_expand")
-
-
-def _lora_call(ys, ds, x, w_a, w_b, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales, plan,
-               name):
-    nproj = len(ys)
-    for i, (y, d) in enumerate(zip(ys, ds)):
-        _check_input(y, f"y[{i}]")
-        _check_input(d, f"delta[{i}]")
-        _check_dim(2, y, f"y[{i}]")
-        _check_dim(2, d, f"delta[{i}]")
-    _check_input(x, "x")
-    _check_dim(2, x, "x")
-    _validate_common(w_a, start_indicies, lora_ranks, loc_indicies, indicies, lora_scales)
-    _check_input(w_b, "w_b")
-    _check_dim(3, w_b, "w_b")
-    batch, h_in, d_cols = x.size(0), x.size(1), ds[0].size(1)
-    if indicies.size(0) != batch:
-        raise RuntimeError(f"CHECK_EQ(indicies.size(0), x.size(0)) failed. {indicies.size(0)} vs {batch}")
-    for i, (y, d) in enumerate(zip(ys, ds)):
-        if d.size(0) != batch or d.size(1) != d_cols or d.dtype != x.dtype:
-            raise RuntimeError(f"delta[{i}] must be [{batch}, {d_cols}] {x.dtype}")
-        if y.size(0) != batch or y.dtype != x.dtype:
-            raise RuntimeError(f"y[{i}] must have {batch} rows of {x.dtype}")
-    no_kernel = f"No suitable kernel. h_in={h_in} h_out={ys[0].size(1)} dtype={x.dtype}"
-    if x.dtype not in (torch.float16, torch.bfloat16) or w_a.dtype != x.dtype or w_b.dtype != x.dtype:
-        raise RuntimeError(no_kernel)
-    if w_a.shape != w_b.shape:
-        raise RuntimeError("the A and B pools must have one shape")
-    if not (h_in >= d_cols and all(d_cols < y.size(1) for y in ys)):
-        raise RuntimeError("delta must be no wider than x and narrower than every y (shrink then expand)")
-    stream = _stream(x)
-    if plan is None:
-        plan = _auto_plan(start_indicies, lora_ranks, loc_indicies, indicies, d_cols, w_a.size(0), stream)
-    if plan is None or plan is False:
-        return False
-    if plan.batch != batch:
-        raise RuntimeError(f"plan was built for {plan.batch} tokens, this call has {batch}")
-    lib = _cabi.load_library()
-    tables = _tables(start_indicies, lora_ranks, loc_indicies)
-    dp = [d.data_ptr() for d in ds] + [None] * (3 - nproj)
-    yp = [y.data_ptr() for y in ys] + [None] * (3 - nproj)
-    hs = [y.size(1) for y in ys] + [0] * (3 - nproj)
-    rc = lib.slora_bgmv_lora_planned(plan.buf.data_ptr(), plan.rank_cap, plan.n_items, nproj, *dp, *yp, x.data_ptr(),
-                                     w_a.data_ptr(), w_b.data_ptr(), C.byref(tables), indicies.data_ptr(),
-                                     lora_scales.data_ptr(), _DTYPE_CODE[lora_scales.dtype], batch, h_in, d_cols,
-                                     *hs, w_a.size(1) * w_a.size(2), w_a.size(0), int(qkvo), _DTYPE_CODE[x.dtype],
-                                     stream)
-    if rc == _cabi.ERR_UNSUPPORTED and h_in > 16384:
-        return False
-    if rc == _cabi.ERR_UNSUPPORTED:
-        raise RuntimeError(no_kernel)
-    _cabi.check(rc, name)
-    return True
-
-
-def dispatch_bgmv_lora(y, delta, x, w_a, w_b, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales,
-                       plan=None) -> None:
-    """The reference's pair of calls for one projection
-    (lora_unordered_batch_infer.py:267-273, 428-448)::
-
-        dispatch_bgmv(delta, x, w_a, ..., qkvo, lora_scales)     # shrink through key_buffer[l]
-        dispatch_bgmv(y, delta, w_b, ..., qkvo, lora_scales)     # expand through value_buffer[l]
-
-    as one launch; same results bit for bit.  Needs a plan (given, or the one
-    kept for these index tensors); without one (graph capture with no ``plan=``,
-    cache off) the two calls are issued."""
-    if not _lora_call([y], [delta], x, w_a, w_b, start_indicies, lora_ranks, loc_indicies, indicies, qkvo,
-                      lora_scales, plan, "dispatch_bgmv_lora"):
-        dispatch_bgmv(delta, x, w_a, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales,
-                      plan=False)
-        dispatch_bgmv(y, delta, w_b, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales,
-                      plan=False)
-
-
-def dispatch_bgmv_qkv_lora(y_q, y_k, y_v, d_q, d_k, d_v, x, w_a, w_b, start_indicies, lora_ranks, loc_indicies,
-                           indicies, lora_scales, plan=None) -> None:
-    """q, k and v of one layer, shrink and expand, as one launch
-    (lora_unordered_batch_infer.py:254-318)."""
-    if not _lora_call([y_q, y_k, y_v], [d_q, d_k, d_v], x, w_a, w_b, start_indicies, lora_ranks, loc_indicies,
-                      indicies, 0, lora_scales, plan, "dispatch_bgmv_qkv_lora"):
-        dispatch_bgmv_qkv_shrink(d_q, d_k, d_v, x, w_a, start_indicies, lora_ranks, loc_indicies, indicies,
-                                 plan=False)
-        dispatch_bgmv_qkv_expand(y_q, y_k, y_v, d_q, d_k, d_v, w_b, start_indicies, lora_ranks, loc_indicies,
-                                 indicies, lora_scales, plan=False)
-
-
-def plan_wait_timed_out(plan) -> bool:
-    """True if a wavefront of a shared shrink + expand launch ever gave up waiting
-    for its run's shrink (never expected; a synchronising read, for tests)."""
-    lib = _cabi.load_library()
-    nbytes = lib.slora_bgmv_plan_bytes(plan.batch, plan.rank_cap)
-    sync0 = int(nbytes) // 4 - (4 + 8 * plan.batch)
-    return bool(int(plan.buf[sync0 + 1].item()))

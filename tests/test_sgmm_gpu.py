@@ -138,7 +138,8 @@ def test_full_size_c3_against_dense_and_decode(gpu):
     atol 1e-3 for the shrink output, 2e-2 for y, which is a bf16 sum of order-1
     terms that may cancel), zero-fill of the columns beyond each rank, and rows
     that belong to no request left alone."""
-    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand, workloads
+    import workloads
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_expand
     w, seg = workloads.c3_prefill(gpu, n_layers=1)
     T, H, R = seg.n_tokens, w.hidden, w.max_rank
     g = torch.Generator(device=gpu)
