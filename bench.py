@@ -58,6 +58,9 @@ def parse_args():
     ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
                     help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="leave out the 'modes' (reference call pattern, direct launches) and 'prefill_c3' blocks "
+                         "that the default S2 run adds to its line")
     ap.add_argument("--cpu-reps", type=int, default=0, help="0 = as many as fit in about 15 s")
     ap.add_argument("--check", action="store_true", help="verify layer 0 against the oracle before timing")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -277,8 +280,66 @@ def cpu_baseline(w, bufs, torch, reps_arg):
 MFMA_PEAK_TFLOPS = 2500.0
 
 
-def main_prefill(args, torch, device):
-    """C3: q/k/v/o segmented shrink and expand over a prefill batch, per layer."""
+def measure_dropin_direct(w, bufs, torch, args):
+    """What an unmodified caller of the reference's engine gets: its call pattern (8
+    stateless-looking dispatch_bgmv calls per layer, new index tensor every step), issued as
+    plain Python calls into the extension, no graph, no plan argument -- the library keeps
+    the plan of the step by itself.  Wall clock around K steps (the launches are asynchronous,
+    so this is the larger of host issue time and device time), and the host cost of one call
+    measured on a one-token batch whose kernels the device finishes faster than they are
+    issued."""
+    import slora_hip
+    t = (w.a_start, w.a_len, w.a_loc)
+    L = w.n_layers
+
+    def step():
+        bins = w.req_bins.clone()  # the engine builds req_bins anew for every step (lora_unordered_batch_infer.py:24)
+        for l in range(L):
+            for p in range(3):
+                slora_hip.dispatch_bgmv(bufs.delta[p], bufs.x_in[l], w.key_buffer[l], *t, bins, p, w.a_scaling)
+                slora_hip.dispatch_bgmv(bufs.y[l][p], bufs.delta[p], w.value_buffer[l], *t, bins, p, w.a_scaling)
+            slora_hip.dispatch_bgmv(bufs.delta[0], bufs.x_att[l], w.key_buffer[l], *t, bins, 3, w.a_scaling)
+            slora_hip.dispatch_bgmv(bufs.y[l][3], bufs.delta[0], w.value_buffer[l], *t, bins, 3, w.a_scaling)
+
+    def wall_ms(fn, n, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / n
+
+    ms = wall_ms(step, max(5, args.steps // 2), 3)
+    # host cost of a call: one token, so the device is never the bottleneck
+    one = torch.zeros(1, dtype=torch.int64, device=w.req_bins.device)
+    x1, d1 = bufs.x_in[0][:1], bufs.delta[0][:1]
+
+    def calls():
+        for _ in range(1000):
+            slora_hip.dispatch_bgmv(d1, x1, w.key_buffer[0], *t, one, 0, w.a_scaling)
+
+    host_us = wall_ms(calls, 3, 1)  # ms per 1000 calls = us per call
+    return {"dropin-direct-autoplan": {
+        "what": "reference call pattern (8 dispatch_bgmv per layer, new req_bins per step), direct launches from "
+                "Python through the extension, plan built and reused by the library",
+        "ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1), "launches_per_step": 8 * L + 2,
+        "host_us_per_call": round(host_us, 2)}}
+
+
+def free_workload(w, bufs, torch):
+    """Give the decode pools back before another workload is built."""
+    w.key_buffer.clear()
+    w.value_buffer.clear()
+    for name in ("x_in", "x_att", "y", "delta"):
+        getattr(bufs, name).clear()
+    torch.cuda.empty_cache()
+
+
+def measure_prefill(args, torch, device):
+    """C3: q/k/v/o segmented shrink and expand over a prefill batch, per layer.  Returns the
+    JSON object of the prefill workload."""
     import slora_hip
     import workloads
     L = min(args.layers, 4)
@@ -346,7 +407,7 @@ def main_prefill(args, torch, device):
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"]},
         "kernels": kernels,
     }
-    print(json.dumps(out), flush=True)
+    return out
 
 
 def main_load(args, torch, device):
@@ -468,7 +529,7 @@ def main():
         del src, dst
 
     if args.workload == "c3":
-        main_prefill(args, torch, device)
+        print(json.dumps(measure_prefill(args, torch, device)), flush=True)
         return
     if args.workload == "load":
         main_load(args, torch, device)
@@ -573,10 +634,16 @@ def main():
         },
         "kernels": kernels,
     }
-    if other_modes:
-        out["modes"] = other_modes
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, bufs, torch, args.cpu_reps)
+    if args.workload == "s2" and not args.no_extras:
+        other_modes.update(measure_dropin_direct(w, bufs, torch, args))
+        free_workload(w, bufs, torch)
+        c3 = measure_prefill(argparse.Namespace(layers=2, steps=10, warmup=3, launch="graph"), torch, device)
+        out["prefill_c3"] = {"tokens_per_s_per_layer": c3["value"], "ms_per_layer": round(c3["ms_per_step"] / 2, 4),
+                             "tokens": c3["config"]["tokens"], "dtype": "bf16", "kernels": c3["kernels"]}
+    if other_modes:
+        out["modes"] = other_modes
     print(json.dumps(out), flush=True)
 
 

@@ -1,7 +1,8 @@
-"""Build libslora_hip.so (HIP kernels + C ABI) for gfx950 with hipcc.
+"""Build libslora_hip.so (HIP kernels + C ABI) for gfx950 with hipcc, and the
+PyTorch extension ``slora_hip/_kernels*.so`` that calls it.
 
-Usage: ``python s-lora_amd/build.py``.  The library lands in
-``s-lora_amd/lib/`` next to the sources, so it travels with the tree.
+Usage: ``python s-lora_amd/build.py``.  Both land in the tree next to the
+sources (``s-lora_amd/lib/`` and ``s-lora_amd/slora_hip/``), so they travel with it.
 """
 from __future__ import annotations
 
@@ -67,6 +68,35 @@ def build_library(verbose: bool = True) -> str:
     return LIB_PATH
 
 
+def extension_path() -> str:
+    import sysconfig
+    return os.path.join(HERE, "slora_hip", "_kernels" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_extension(verbose: bool = True) -> str:
+    """Compile csrc/torch_ext.cpp (host code only: pybind11 + tensor checks + calls into
+    the C ABI) against this interpreter's torch and link it to libslora_hip.so."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build_library() first")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    out = extension_path()
+    cmd = [hipcc_path(), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall",
+           "-Wno-unused-function", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_kernels",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I", os.path.join(ROOT, "include"), "-I", sysconfig.get_paths()["include"]]
+    for inc in cpp_extension.include_paths():
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(CSRC, "torch_ext.cpp"), "-o", out,
+            "-L", torch_lib, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+            "-L", LIB_DIR, "-lslora_hip", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,--no-as-needed"]
+    _run(cmd, verbose)
+    return out
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_extension(verbose=True))
     sys.exit(0)

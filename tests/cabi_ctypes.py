@@ -1,12 +1,13 @@
-"""ctypes binding of libslora_hip.so (the declarations of include/slora_hip.h)."""
+"""ctypes binding of libslora_hip.so (the declarations of include/slora_hip.h), for the tests
+that call the C ABI directly.  The product binds the same functions from C++
+(s-lora_amd/csrc/torch_ext.cpp)."""
 from __future__ import annotations
 
 import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# SLORA_HIP_LIB names another build of the same library (e.g. one compiled with other tuning constants)
-_LIB_PATH = os.environ.get("SLORA_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libslora_hip.so")
+_LIB_PATH = os.path.join(os.path.dirname(_HERE), "s-lora_amd", "lib", "libslora_hip.so")
 
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 MAX_RANK = 512  # SLORA_MAX_RANK of include/slora_hip.h

@@ -19,15 +19,16 @@ TDT = {"f16": torch.float16, "bf16": torch.bfloat16}
 
 
 @pytest.fixture(autouse=True, params=["cache", "stateless"])
-def plan_cache_mode(request, monkeypatch):
+def plan_cache_mode(request):
     """Every test runs twice: with calls that pass no plan served by the
     automatic plan cache (the default), and with the cache off, which sends the
     same calls to the kernels that find their runs by themselves."""
     import slora_hip
-    monkeypatch.setenv("SLORA_PLAN_CACHE", "1" if request.param == "cache" else "0")
+    slora_hip.set_plan_cache_enabled(request.param == "cache")
     slora_hip.clear_plan_cache()
     yield request.param
     slora_hip.clear_plan_cache()
+    slora_hip.set_plan_cache_enabled(True)
 
 
 def dev(a, dtype, device):
@@ -366,13 +367,17 @@ def test_automatic_plan_cache_follows_the_index_tensors(gpu, plan_cache_mode):
     """Calls without a plan reuse one built at the first call for the same index
     tensors; an in-place change of a tensor or a new tensor object rebuilds it,
     and the results always equal those of the plan-free kernels."""
-    from slora_hip import dispatch_bgmv, _kernels
+    import slora_hip
+    from slora_hip import dispatch_bgmv
     if plan_cache_mode != "cache":
         pytest.skip("cache switched off")
     c = make_case(77, 512, [16, 8, 32], 40, dtype="f16")
     g = GpuCase(c, gpu)
-    cache = _kernels._plan_cache
-    cache.hits = cache.builds = 0
+    slora_hip.plan_cache_stats(reset=True)
+
+    def stats():
+        s = slora_hip.plan_cache_stats()
+        return s["builds"], s["hits"]
 
     def both(bins):
         t = (g.a_start, g.a_len, g.a_loc, bins)
@@ -388,18 +393,45 @@ def test_automatic_plan_cache_follows_the_index_tensors(gpu, plan_cache_mode):
         assert torch.equal(y0, y1)
 
     both(g.bins)
-    assert (cache.builds, cache.hits) == (1, 1)   # shrink built it, expand reused it
+    assert stats() == (1, 1)                       # shrink built it, expand reused it
     both(g.bins)
-    assert (cache.builds, cache.hits) == (1, 3)
+    assert stats() == (1, 3)
     g.bins.copy_(torch.flip(g.bins, dims=[0]))     # new batch written in place: version changes
     both(g.bins)
-    assert cache.builds == 2
+    assert stats()[0] == 2
     both(g.bins.clone())                           # same contents in a new tensor object
-    assert cache.builds == 3
+    assert stats()[0] == 3
     torch.cuda.synchronize()
     with torch.cuda.stream(torch.cuda.Stream()):   # another stream never sees this stream's plan
         both(g.bins)
-    assert cache.builds == 4
+    assert stats()[0] == 4
+    # a new tensor object that lands at the address (and version) of a freed one is another tensor
+    slora_hip.clear_plan_cache()
+    slora_hip.plan_cache_stats(reset=True)
+    for k in range(3):
+        b = torch.roll(g.bins, k).contiguous()
+        both(b)
+        del b
+    assert stats()[0] == 3
+    # a table rewritten through this library's own raw-pointer writers invalidates the plan
+    from slora_hip.infer_adapter import launch_var_len_copy
+    slora_hip.clear_plan_cache()
+    slora_hip.plan_cache_stats(reset=True)
+    loc = g.a_loc.clone()
+    t2 = (g.a_start, g.a_len, loc, g.bins)
+    d_a = torch.zeros((c.batch, 32), dtype=g.tdt, device=gpu)
+    dispatch_bgmv(d_a, g.x, g.key, *t2, 1, g.scales)
+    # move every adapter's page list to where another adapter's was: same tensor object, new contents
+    new_loc = torch.flip(g.a_loc, dims=[0]).contiguous()
+    launch_var_len_copy(torch.zeros(1, dtype=torch.int64, device=gpu),
+                        torch.full((1,), loc.numel(), dtype=torch.int64, device=gpu), new_loc,
+                        torch.zeros(1, dtype=torch.int64, device=gpu), loc)
+    d_b = torch.zeros_like(d_a)
+    dispatch_bgmv(d_b, g.x, g.key, *t2, 1, g.scales)
+    d_c = torch.zeros_like(d_a)
+    dispatch_bgmv(d_c, g.x, g.key, *t2, 1, g.scales, plan=False)
+    assert torch.equal(d_b, d_c) and not torch.equal(d_a, d_b)
+    assert stats()[0] == 2
 
 
 @pytest.mark.parametrize("seed", range(12))

@@ -12,15 +12,15 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 @pytest.fixture(scope="module")
 def lib():
-    import slora_hip
-    from slora_hip import _cabi
+    import cabi_ctypes as _cabi
     if not os.path.exists(_cabi.lib_path()):
         import importlib.util
         spec = importlib.util.spec_from_file_location("slora_build", os.path.join(ROOT, "s-lora_amd", "build.py"))
         mod = importlib.util.module_from_spec(spec)
         spec.loader.exec_module(mod)
         mod.build_library(verbose=False)
-    return slora_hip.load_library()
+        mod.build_extension(verbose=False)
+    return _cabi.load_library()
 
 
 def declared_functions():
@@ -30,7 +30,7 @@ def declared_functions():
 
 
 def test_header_and_binding_agree(lib):
-    from slora_hip import _cabi
+    import cabi_ctypes as _cabi
     names = declared_functions()
     assert names == sorted(_cabi.SIGNATURES)
     for n in names:
@@ -38,7 +38,7 @@ def test_header_and_binding_agree(lib):
 
 
 def test_version_and_strerror(lib):
-    from slora_hip import _cabi
+    import cabi_ctypes as _cabi
     assert lib.slora_version() == 100
     assert _cabi.strerror(0) == "ok"
     assert "No suitable kernel" in _cabi.strerror(_cabi.ERR_UNSUPPORTED)
@@ -48,12 +48,12 @@ def test_version_and_strerror(lib):
 
 
 def _tables(ptr=0x1000):
-    from slora_hip import _cabi
+    import cabi_ctypes as _cabi
     return _cabi.SloraTables(ptr, ptr, ptr, 4, 64)
 
 
 def test_shrink_argument_checks(lib):
-    from slora_hip import _cabi as A
+    import cabi_ctypes as A
     t = _tables()
     P = 0x10000  # never dereferenced: every call below fails validation or has nothing to do
     f = lib.slora_bgmv_shrink
@@ -72,7 +72,7 @@ def test_shrink_argument_checks(lib):
 
 
 def test_expand_argument_checks(lib):
-    from slora_hip import _cabi as A
+    import cabi_ctypes as A
     t = _tables()
     P = 0x10000
     f = lib.slora_bgmv_expand
@@ -85,7 +85,7 @@ def test_expand_argument_checks(lib):
 
 
 def test_sgmm_argument_checks(lib):
-    from slora_hip import _cabi as A
+    import cabi_ctypes as A
     t = _tables()
     P = 0x10000
     s = lib.slora_sgmm_shrink

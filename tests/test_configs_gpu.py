@@ -29,14 +29,15 @@ RTOL, ATOL = 1e-2, 1e-3
 
 
 @pytest.fixture(params=["cache", "stateless"])
-def plan_cache_mode(request, monkeypatch):
+def plan_cache_mode(request):
     """Calls that pass no plan are served by the automatic plan cache (the default) or,
     with the cache off, by the kernels that find their runs by themselves."""
     import slora_hip
-    monkeypatch.setenv("SLORA_PLAN_CACHE", "1" if request.param == "cache" else "0")
+    slora_hip.set_plan_cache_enabled(request.param == "cache")
     slora_hip.clear_plan_cache()
     yield request.param
     slora_hip.clear_plan_cache()
+    slora_hip.set_plan_cache_enabled(True)
 
 
 # ---------------------------------------------------------------------------

@@ -12,15 +12,16 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(autouse=True, params=["cache", "no-plan"])
-def prefill_plan_mode(request, monkeypatch):
+def prefill_plan_mode(request):
     """Every test runs twice: with shrink calls served by the automatic per-batch plan
     (the default) and with the cache off, which sends them to the kernel that works out
     its share of the batch by itself."""
     import slora_hip
-    monkeypatch.setenv("SLORA_PLAN_CACHE", "1" if request.param == "cache" else "0")
+    slora_hip.set_plan_cache_enabled(request.param == "cache")
     slora_hip.clear_prefill_plan_cache()
     yield request.param
     slora_hip.clear_prefill_plan_cache()
+    slora_hip.set_plan_cache_enabled(True)
 
 
 def seg_case(seed, hidden, ranks, n_req, lo, hi, dtype, h_out=None, sort=True):
@@ -299,15 +300,19 @@ def test_prefill_plan_gives_the_plain_kernels_bits(gpu, hidden, ranks, n_req, lo
 
 
 def test_prefill_plan_cache_follows_the_index_tensors(gpu, prefill_plan_mode):
-    from slora_hip import lora_get_qkvo_fwd_shrink, lora_prefill
+    import slora_hip
+    from slora_hip import lora_get_qkvo_fwd_shrink
     if prefill_plan_mode != "cache":
         pytest.skip("cache switched off")
     c = seg_case(31, 256, [16, 8, 32], 12, 1, 90, "f16")
     g = GpuCase(c, gpu)
     start, lens, ids, max_len = _shrink_args(c, g, gpu)
     w_a = g.key.view(c.n_pages, c.page_elems)
-    cache = lora_prefill._prefill_plan_cache
-    cache.hits = cache.builds = 0
+    slora_hip.plan_cache_stats(reset=True)
+
+    def stats():
+        s = slora_hip.plan_cache_stats()
+        return s["prefill_builds"], s["prefill_hits"]
 
     def both(lens_t, ids_t):
         o0 = torch.full((c.batch, 32), 3.0, dtype=g.tdt, device=gpu)  # rows of no request keep this value
@@ -321,20 +326,23 @@ def test_prefill_plan_cache_follows_the_index_tensors(gpu, prefill_plan_mode):
 
     both(lens, ids)
     both(lens, ids)
-    assert (cache.builds, cache.hits) == (1, 1)
+    assert stats() == (1, 1)
     ids.copy_(torch.flip(ids, dims=[0]))          # in place: the version changes, the plan is rebuilt
     both(lens, ids)
-    assert cache.builds == 2
+    assert stats()[0] == 2
     lens2 = lens.clone()                          # another object with the same values: rebuilt as well
     both(lens2, ids)
-    assert cache.builds == 3
+    assert stats()[0] == 3
     lens2[0] = 0                                  # a request dropped in place
     both(lens2, ids)
-    assert cache.builds == 4
+    assert stats()[0] == 4
     # a caller that makes new tensors for every call gets no plan after a few useless builds
-    for _ in range(cache.MISS_STREAK + 3):
+    for _ in range(8 + 3):
         both(lens2.clone(), ids)
-    assert cache.paused > 0 and cache.builds <= 4 + cache.MISS_STREAK
+    assert stats()[0] <= 4 + 8
+    built = stats()[0]
+    both(lens2.clone(), ids)                      # paused: no build
+    assert stats()[0] == built
 
 
 def test_prefill_plan_of_another_batch_is_rejected(gpu):
