@@ -50,6 +50,7 @@ extern "C" {
 #define SLORA_ERR_UNSUPPORTED -4   /* "No suitable kernel": width not a multiple of 8, rank above 512, ... */
 #define SLORA_ERR_ALIGNMENT -5     /* a buffer the kernels read 16 bytes at a time is not 16-byte aligned */
 #define SLORA_ERR_LAUNCH -6        /* the HIP runtime refused the launch */
+#define SLORA_ERR_TOO_LARGE -7     /* a size exceeds the fixed capacity of an entry point that allocates nothing */
 
 #define SLORA_MAX_RANK 512
 
@@ -286,6 +287,18 @@ SLORA_API int slora_pool_alloc(uint8_t* mem_state, int64_t tot_size, int64_t nee
  * result[1] = pages handed out. */
 SLORA_API int slora_pool_alloc_contiguous(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index,
                                 int64_t* result, void* workspace, void* stream);
+
+/* slora_pool_alloc_contiguous without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops and
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * workspace is an array inside the library's device image (about 48 KiB, held by
+ * every GPU the library runs on until the process ends), good for maps of up to
+ * SLORA_POOL_STATIC_MAX_PAGES pages; a larger tot_size returns SLORA_ERR_TOO_LARGE.
+ * Arguments and results are those of slora_pool_alloc_contiguous.  All calls on
+ * one GPU share the array: calls that overlap on one GPU (two streams) race. */
+#define SLORA_POOL_STATIC_MAX_PAGES (1 << 24)
+SLORA_API int slora_pool_alloc_contiguous_static(uint8_t* mem_state, int64_t tot_size, int64_t need,
+                                                 int64_t* out_index, int64_t* result, void* stream);
 
 /* MemoryAllocator.free (mem_allocator.py:185-199): mem_state[free_index] = 1;
  * ids outside the map are skipped. */

@@ -14,6 +14,7 @@ const char* slora_strerror(int code) {
     case SLORA_ERR_UNSUPPORTED: return "No suitable kernel.";
     case SLORA_ERR_ALIGNMENT: return "buffer is not 16-byte aligned";
     case SLORA_ERR_LAUNCH: return "HIP kernel launch failed";
+    case SLORA_ERR_TOO_LARGE: return "size exceeds the fixed capacity of this entry point (see its maximum in slora_hip.h)";
     default: return "unknown error";
   }
 }

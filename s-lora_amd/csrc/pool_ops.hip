@@ -20,11 +20,50 @@
 // All of it is plain byte/integer movement, bound by HBM bandwidth (the first) or
 // by a handful of dependent round trips (the rest).
 
+#include <mutex>
+
 #include "common.hpp"
 #include "cabi_util.hpp"
 
 namespace slora {
 namespace {
+
+// ---------------------------------------------------------------------------
+// workspace of slora_pool_alloc_contiguous_static
+// ---------------------------------------------------------------------------
+// The allocator's workspace (best start, per-workgroup free counts and last used
+// pages) for maps of up to kStaticMapPages pages, held by every GPU the library
+// runs on until the process ends.  In host code the array's name is only a
+// handle: the address the kernels get comes from hipGetSymbolAddress, once per
+// device, with that device current (every GPU has its own copy at its own
+// address).
+constexpr int64_t kStaticMapPages = int64_t(1) << 24;  // 16 Mi pages: 128 GiB of 8 KiB pages
+constexpr int64_t kStaticMapBlocks = kStaticMapPages / (256 * 16);
+constexpr int64_t kStaticScratchBytes = 16 + kStaticMapBlocks * 4 + 8 + kStaticMapBlocks * 8;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices];  // per device: the address of `scratch` there, nullptr = not asked yet
+
+// the current device's copy of `scratch`, or nullptr if the runtime cannot name it
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
 
 // ---------------------------------------------------------------------------
 // scatter rows into pool pages
@@ -605,6 +644,20 @@ int slora_pool_alloc_contiguous(uint8_t* mem_state, int64_t tot_size, int64_t ne
   hipLaunchKernelGGL(map_take_run_kernel, dim3((uint32_t)grid), dim3(kMapThreads), 0, s, mem_state, tot_size, need,
                      best, out_index, result);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_alloc_contiguous_static(uint8_t* mem_state, int64_t tot_size, int64_t need, int64_t* out_index,
+                                       int64_t* result, void* stream) {
+  using namespace slora;
+  if (tot_size > kStaticMapPages) return SLORA_ERR_TOO_LARGE;
+  static_assert(kStaticMapBlocks * kMapBlock == kStaticMapPages, "the static workspace is sized in whole map blocks");
+  static_assert(kStaticMapPages == SLORA_POOL_STATIC_MAX_PAGES, "the header states the capacity");
+  if (tot_size >= 0 && slora_pool_alloc_workspace_bytes(tot_size) > kStaticScratchBytes) return SLORA_ERR_TOO_LARGE;
+  void* ws = static_scratch();
+  if (ws == nullptr) return SLORA_ERR_LAUNCH;
+  // same kernels as slora_pool_alloc_contiguous; its first launch resets the best start, and the
+  // per-workgroup entries it reads are all rewritten by the launch in front of the reader
+  return slora_pool_alloc_contiguous(mem_state, tot_size, need, out_index, result, ws, stream);
 }
 
 int slora_pool_free(uint8_t* mem_state, int64_t tot_size, const int64_t* free_index, int64_t n, void* stream) {

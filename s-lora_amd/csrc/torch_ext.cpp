@@ -795,14 +795,20 @@ void pool_alloc(const Tensor& mem_state, int64_t need, const Tensor& out_index, 
 }
 
 void pool_alloc_contiguous(const Tensor& mem_state, int64_t need, const Tensor& out_index, const Tensor& result,
-                           const Tensor& work) {
+                           const c10::optional<Tensor>& work) {
   check_map(mem_state);
   TORCH_CHECK(out_index.is_cuda() && out_index.scalar_type() == at::kLong && out_index.numel() >= need, "out_index must hold `need` int64");
   TORCH_CHECK(result.is_cuda() && result.scalar_type() == at::kLong && result.numel() >= 2, "result must hold two int64");
-  TORCH_CHECK(work.is_cuda() && work.nbytes() >= (size_t)slora_pool_alloc_workspace_bytes(mem_state.numel()), "workspace too small");
-  const int rc = slora_pool_alloc_contiguous(static_cast<uint8_t*>(mem_state.data_ptr()), mem_state.numel(), need,
-                                             out_index.data_ptr<int64_t>(), result.data_ptr<int64_t>(), work.data_ptr(),
-                                             stream_of(mem_state));
+  int rc;
+  if (work.has_value()) {
+    TORCH_CHECK(work->is_cuda() && work->nbytes() >= (size_t)slora_pool_alloc_workspace_bytes(mem_state.numel()), "workspace too small");
+    rc = slora_pool_alloc_contiguous(static_cast<uint8_t*>(mem_state.data_ptr()), mem_state.numel(), need,
+                                     out_index.data_ptr<int64_t>(), result.data_ptr<int64_t>(), work->data_ptr(),
+                                     stream_of(mem_state));
+  } else {  // the library's own static workspace: nothing allocated
+    rc = slora_pool_alloc_contiguous_static(static_cast<uint8_t*>(mem_state.data_ptr()), mem_state.numel(), need,
+                                            out_index.data_ptr<int64_t>(), result.data_ptr<int64_t>(), stream_of(mem_state));
+  }
   check_rc(rc, "PageAllocator.alloc_contiguous");
   mark_written(mem_state);
   mark_written(out_index);
@@ -900,7 +906,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("compact_adapter_tables_raw", &compact_adapter_tables_raw);
   m.def("pool_alloc_workspace_bytes", &pool_alloc_workspace_bytes);
   m.def("pool_alloc", &pool_alloc);
-  m.def("pool_alloc_contiguous", &pool_alloc_contiguous);
+  m.def("pool_alloc_contiguous", &pool_alloc_contiguous, py::arg("mem_state"), py::arg("need"), py::arg("out_index"),
+        py::arg("result"), py::arg("work") = py::none());
   m.def("pool_free", &pool_free);
   m.def("gather_lora_a", &gather_lora_a, py::arg("key_buffer"), py::arg("a_loc"), py::arg("first"), py::arg("rank"),
         py::arg("hidden"), py::arg("out_cols") = 0);

@@ -13,7 +13,8 @@ DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 MAX_RANK = 512  # SLORA_MAX_RANK of include/slora_hip.h
 
 OK = 0
-ERR_NULL_POINTER, ERR_BAD_DTYPE, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_ALIGNMENT, ERR_LAUNCH = -1, -2, -3, -4, -5, -6
+ERR_NULL_POINTER, ERR_BAD_DTYPE, ERR_BAD_SHAPE, ERR_UNSUPPORTED, ERR_ALIGNMENT, ERR_LAUNCH, ERR_TOO_LARGE = \
+    -1, -2, -3, -4, -5, -6, -7
 
 
 class SloraTables(C.Structure):
@@ -59,6 +60,7 @@ SIGNATURES = {
     "slora_pool_alloc_workspace_bytes": (_I64, [_I64]),
     "slora_pool_alloc": (_I, [_P, _I64, _I64, _P, _P, _P, _P]),
     "slora_pool_alloc_contiguous": (_I, [_P, _I64, _I64, _P, _P, _P, _P]),
+    "slora_pool_alloc_contiguous_static": (_I, [_P, _I64, _I64, _P, _P, _P]),
     "slora_pool_free": (_I, [_P, _I64, _P, _I64, _P]),
 }
 

@@ -42,7 +42,7 @@ def test_version_and_strerror(lib):
     assert lib.slora_version() == 100
     assert _cabi.strerror(0) == "ok"
     assert "No suitable kernel" in _cabi.strerror(_cabi.ERR_UNSUPPORTED)
-    for code in range(-6, 0):
+    for code in range(-7, 0):
         assert _cabi.strerror(code) != "unknown error"
     assert _cabi.strerror(-99) == "unknown error"
 
