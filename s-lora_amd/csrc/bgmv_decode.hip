@@ -211,7 +211,7 @@ struct ShrinkArgs {
   const int* plan;  // nullptr: stateless
   Tables t;
   int64_t page_elems;
-  int batch, h_in, y_cols, qkvo0, blocks, lds_tt, units;
+  int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
 };
 
 // The common case in straight-line code: hidden <= 4096 (one pass), all tokens
@@ -296,12 +296,13 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 }
 
 // 4 wavefronts; wavefront w takes rows j0+w and j0+w+4 of one projection.  A
-// q/k/v call launches three workgroups per item (projection-major, so that with
-// a multiple of 8 items all three run on the item's XCD and share its
-// activations in that L2).
-// `block` = projection * units + item.  s_x: [lds_tt][h_in / 8] LDS words.
+// q/k/v call launches three workgroups per item (grid y = projection: workgroup ids
+// run item-fastest, so with a multiple of 8 items all three land on the item's XCD
+// and share its activations in that L2).
+// Grid: x = item (planned) or token * blocks + block (stateless), y = projection of the
+// launch.  s_x: [lds_tt][h_in / 8] LDS words.
 template <typename T, bool PLANNED>
-__device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x4* s_x) {
+__device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int proj, u32x4* s_x) {
   constexpr int NW = 4;
   constexpr int NTASK = 2;
   constexpr int NT = NW * kWave;
@@ -309,8 +310,6 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  const int proj = block / p.units;
-  const int unit = block - proj * p.units;
   Item it;
   const int* rec = PLANNED ? p.plan + kPlanHeaderWords + (int64_t)unit * kItemWords : nullptr;
   int plan_pg0 = -1, plan_pg1 = -1;
@@ -459,7 +458,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int block, u32x
 template <typename T, bool PLANNED>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];  // [lds_tt][h_in / 8]
-  shrink_body<T, PLANNED>(p, (int)blockIdx.x, s_x);
+  shrink_body<T, PLANNED>(p, (int)blockIdx.x, (int)blockIdx.y, s_x);
 }
 
 // ---------------------------------------------------------------------------
@@ -474,23 +473,63 @@ struct ExpandArgs {
   Tables t;
   int64_t page_elems;
   int scales_dtype;
-  int batch, x_cols, qkvo0, blocks, y_aligned, units;
+  int batch, x_cols, qkvo0, blocks, y_aligned;
   int h_out[3];
+  // pages per rank row of each projection: a rank-r adapter's B^T fills ceil(r * h_out /
+  // page_elems) pages.  pages_shift >= 0: page_elems = h_out << pages_shift (the count is a
+  // shift); -1: h_out >= page_elems (all r pages); -2: neither (a division on the device).
+  int pages_shift[3];
 };
 
-// Reduce the 8 partial sums of a pass over the LPO lanes that share an output
-// and file them, rounded to the storage type, in the wavefront's LDS strip:
-// load c covers outputs c*OPW .. c*OPW+OPW-1 of the pass, and lane c % LPO of
-// each lane group writes it.
-template <typename T, int LPO>
-__device__ __forceinline__ void file_sums(const float (&part)[kVecPerPass], float scale, int lane, uint16_t* s_strip) {
-  constexpr int OPW = kWave / LPO;
-  const int li = lane % LPO, g = lane / LPO;
+// One exchange of a reduce-scatter over the lanes that share an output: a lane holds N
+// partial sums (one per load of the pass); the lane with `up` keeps the upper N/2 and
+// hands the lower N/2 to its partner, the other lane the reverse, and each adds what it
+// receives to what it keeps.  CTRL is the DPP pattern that names the partner.
+template <int CTRL, int N>
+__device__ __forceinline__ void rs_stage(float (&v)[kVecPerPass], bool up) {
 #pragma unroll
-  for (int c = 0; c < kVecPerPass; ++c) {
-    const float s = group_sum<LPO>(part[c]);
-    if (li == (c % LPO)) s_strip[c * OPW + g] = T::from_float(s * scale);
+  for (int i = 0; i < N / 2; ++i) {
+    const float keep = up ? v[i + N / 2] : v[i];
+    const float send = up ? v[i] : v[i + N / 2];
+    const int got = __builtin_amdgcn_update_dpp(0, __float_as_int(send), CTRL, 0xf, 0xf, false);
+    v[i] = keep + __int_as_float(got);
   }
+}
+
+// Sum the 8 partial sums of a pass (one per load) over the LPO lanes that share an
+// output and file them, scaled and rounded to the storage type, in the wavefront's LDS
+// strip at [c * OPW + g] (load c, lane group g): the strip then holds the pass's outputs
+// in order.  The sums are reduce-scattered: every exchange halves what a lane holds, so
+// that the LPO lanes of a group end up with 8 / LPO different loads each (lane li of the
+// group with loads li * 8 / LPO + i) and every lane writes only sums nobody else has.
+// The first exchanges use the mirror patterns (their partners differ in all lower lane
+// bits, which is fine while every lane still holds every load), the last ones xor 2 and
+// xor 1, which keep the upper bits that by then decide what a lane holds.
+template <typename T, int LPO>
+__device__ __forceinline__ void file_sums(float (&v)[kVecPerPass], float scale, int lane, uint16_t* s_strip) {
+  static_assert(LPO == 1 || LPO == 2 || LPO == 4 || LPO == 8 || LPO == 16, "lanes per output");
+  constexpr int OPW = kWave / LPO;
+  constexpr int kRowMirror = 0x140, kHalfMirror = 0x141, kXor2 = 0x4E, kXor1 = 0xB1;
+  if (LPO == 16) {
+    rs_stage<kRowMirror, 8>(v, (lane & 8) != 0);
+    rs_stage<kHalfMirror, 4>(v, (lane & 4) != 0);
+    rs_stage<kXor2, 2>(v, (lane & 2) != 0);
+    v[0] = dpp_add<kXor1>(v[0]);  // both lanes of the last pair hold the sum; either may write it
+  } else if (LPO == 8) {
+    rs_stage<kHalfMirror, 8>(v, (lane & 4) != 0);
+    rs_stage<kXor2, 4>(v, (lane & 2) != 0);
+    rs_stage<kXor1, 2>(v, (lane & 1) != 0);
+  } else if (LPO == 4) {
+    rs_stage<kXor2, 8>(v, (lane & 2) != 0);
+    rs_stage<kXor1, 4>(v, (lane & 1) != 0);
+  } else if (LPO == 2) {
+    rs_stage<kXor1, 8>(v, (lane & 1) != 0);
+  }
+  constexpr int NV = LPO >= 8 ? 1 : kVecPerPass / LPO;  // sums this lane holds now
+  const int li = lane % LPO, g = lane / LPO;
+  const int c0 = LPO == 16 ? li >> 1 : li * NV;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) s_strip[(c0 + i) * OPW + g] = T::from_float(v[i] * scale);
 }
 
 // One page of the flattened (h_out, r) matrix B^T for one run, rank r a power
@@ -499,7 +538,10 @@ __device__ __forceinline__ void file_sums(const float (&part)[kVecPerPass], floa
 // scaled sums of a pass are transposed through a 1 KiB LDS strip of the
 // wavefront so that the read-modify-write of y is one 16-byte load and one
 // 16-byte store per lane and token.
-template <typename T>
+// FULL: every element of the page belongs to an output inside h_out and every rank
+// column is used (the caller checks: whole passes, page inside the output, delta as wide
+// as the rank) -- then no load needs its result masked.
+template <typename T, bool FULL>
 __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const Item& it, int r_eff,
                                             const uint16_t* wpage, int64_t flat0, float scale, uint16_t* s_strip) {
   const int lane = threadIdx.x & 63;
@@ -507,7 +549,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
   const int lg_r = __builtin_ctz((unsigned)r);
   const int lpo = r >> 3;
   const int d0 = (lane & (lpo - 1)) * 8;
-  const bool d_ok = d0 < r_eff;
+  const bool d_ok = FULL || d0 < r_eff;
   const int page_elems = (int)p.page_elems;
   const int out_per_pass = kPassElems >> lg_r;
   const int n_page0 = (int)(flat0 >> lg_r);  // first output of this page
@@ -523,21 +565,33 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
   for (int c = 0; c < kVecPerPass; ++c) {
     const int e = (c * kWave + lane) * 8;
-    const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
-    wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
+    if (FULL) {
+      wv[c] = ldg16_stream(wpage + e);
+    } else {
+      const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
+      wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
+    }
   }
   u32x4 xv[kTT];
 #pragma unroll
-  for (int t = 0; t < kTT; ++t)
-    xv[t] = (t < it.n_tok && d_ok) ? ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0) : zero16();
+  for (int t = 0; t < kTT; ++t) {
+    if (FULL)  // a token the run does not have re-reads the first one's row; its sums are never used
+      xv[t] = ldg16(x + (int64_t)(t < it.n_tok ? it.tok[t] : it.tok[0]) * p.x_cols + d0);
+    else
+      xv[t] = (t < it.n_tok && d_ok) ? ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0) : zero16();
+  }
 
   for (int e0 = 0; e0 < page_elems; e0 += kPassElems) {
     if (e0 != 0) {
 #pragma unroll
       for (int c = 0; c < kVecPerPass; ++c) {
         const int e = e0 + (c * kWave + lane) * 8;
-        const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
-        wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
+        if (FULL) {
+          wv[c] = ldg16_stream(wpage + e);
+        } else {
+          const bool w_ok = d_ok && e < page_elems && n_page0 + (e >> lg_r) < n_end;
+          wv[c] = w_ok ? ldg16_stream(wpage + e) : zero16();
+        }
       }
     }
     // this lane's 8 consecutive outputs of the pass
@@ -546,8 +600,13 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
     u32x4 yv[kTT];
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
-      const uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
-      yv[t] = (t < it.n_tok && y_ok) ? ldg16_stream(yp) : zero16();
+      if (FULL) {  // lanes with no outputs re-read the page's first ones; the values are not used
+        yv[t] = ldg16_stream(y + (int64_t)(t < it.n_tok ? it.tok[t] : it.tok[0]) * h_stride +
+                             (y_ok ? n_mine : n_page0));
+      } else {
+        const uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n_mine;
+        yv[t] = (t < it.n_tok && y_ok) ? ldg16_stream(yp) : zero16();
+      }
     }
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
@@ -567,11 +626,7 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
         if (y_ok) {
           u32x4 out;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint16_t lo = T::add((uint16_t)(yv[t][q] & 0xffffu), (uint16_t)(dv[q] & 0xffffu));
-            const uint16_t hi = T::add((uint16_t)(yv[t][q] >> 16), (uint16_t)(dv[q] >> 16));
-            out[q] = (uint32_t)lo | ((uint32_t)hi << 16);
-          }
+          for (int q = 0; q < 4; ++q) out[q] = T::add2(yv[t][q], dv[q]);
           stg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine, out);
         }
       }
@@ -626,20 +681,26 @@ __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const 
   if (page < 0) return;
   const uint16_t* wpage = reinterpret_cast<const uint16_t*>(p.w) + page * p.page_elems;
   const int64_t flat0 = (int64_t)kk * p.page_elems;
-  expand_page<T>(p, proj, it, r_eff, wpage, flat0, load_scale(p.scales, p.scales_dtype, it.a), s_strip);
+  const float scale = load_scale(p.scales, p.scales_dtype, it.a);
+  // the whole page lies inside the output, in whole passes, and delta is as wide as the rank
+  const bool full = r_eff == it.r && (p.page_elems & (kPassElems - 1)) == 0 &&
+                    flat0 + p.page_elems <= (int64_t)p.h_out[proj] * it.r;
+  if (full)
+    expand_page<T, true>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
+  else
+    expand_page<T, false>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
 }
 
 // Expand has nothing to share between wavefronts (the delta row is 16 bytes per
 // lane), so every wavefront takes exactly one page: a workgroup is 4 wavefronts
 // = half of one projection's 8-page block of an item, and an item gets
 // 2 * NPROJ workgroups.
-// `block` = (projection * 2 + half) * units + item.
+// Grid: x = item (planned) or token * blocks + block (stateless), y = projection * 2 +
+// half: workgroup ids run item-fastest, so with a multiple of 8 items every workgroup of
+// an item lands on XCD item % 8.
 template <typename T, int NPROJ, bool PLANNED>
-__device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint16_t* s_strip) {
+__device__ __forceinline__ void expand_body(const ExpandArgs& p, int unit, int sub, uint16_t* s_strip) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // sub-block major: with a multiple of 8 units, every workgroup of a unit lands on XCD unit % 8
-  const int sub = block / p.units;
-  const int unit = block - sub * p.units;
   const int proj = sub >> 1;
   const int jr = (sub & 1) * 4 + wave;  // page inside the item's block
 
@@ -658,7 +719,14 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint
   if (r_eff <= 0) return;
   const int k = it.j0 + jr;
   // pages that hold this projection's h_out * r elements
-  int64_t n_pg = ((int64_t)p.h_out[proj] * r + p.page_elems - 1) / p.page_elems;
+  const int sh = p.pages_shift[proj];
+  int n_pg = r;
+  if (sh >= 0)
+    n_pg = (r + (1 << sh) - 1) >> sh;
+  else if (sh == -2)
+    n_pg = r > 512 ? (int)(((int64_t)p.h_out[proj] * r + p.page_elems - 1) / p.page_elems)
+                   : (int)(((uint32_t)p.h_out[proj] * (uint32_t)r + (uint32_t)p.page_elems - 1u) /
+                           (uint32_t)p.page_elems);
   if (n_pg > r) n_pg = r;
   // Pages the launch does not enumerate: the stateless grid stops at the delta
   // width and a plan at rank_cap; an adapter of larger rank has more, which
@@ -673,7 +741,7 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int block, uint
   const bool pow2 = (r & (r - 1)) == 0;
   // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
   const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
-                      (p.page_elems % (8 * r)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
+                      (p.page_elems & (8 * r - 1)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
   if (k < n_pg) {
     const int64_t page = PLANNED ? (int64_t)plan_pg : (int64_t)-2;
     expand_one<T>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
@@ -1063,9 +1131,10 @@ constexpr size_t kLdsSoftLimit = 64 * 1024;
 constexpr size_t kLdsHardLimit = 160 * 1024 - 256;
 
 // item capacity of a plan: every run's items plus the padding that evens out the 8 queues
+// (a whole number of groups of 8, so that a launch sized for the capacity keeps item i on XCD i % 8)
 int64_t plan_max_items(int64_t batch, int64_t rank_cap) {
   const int64_t per_run = (rank_cap + kRB - 1) / kRB;
-  return batch * per_run + kXcds * (per_run + 1);
+  return (batch * per_run + kXcds - 1) / kXcds * kXcds + kXcds * (per_run + 1);
 }
 // int32 words of the builder's scratch area behind the items
 int64_t plan_scratch_words(int64_t batch) { return batch * SC_WORDS; }
@@ -1083,8 +1152,7 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
   if (lds > kLdsHardLimit) return SLORA_ERR_UNSUPPORTED;
   p.lds_tt = tt;
   auto kernel = bgmv_shrink_kernel<T, PLANNED>;
-  p.units = (int)units;
-  const int64_t grid = units * nproj;
+  const int64_t grid = units;
   if (lds > kLdsSoftLimit) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess) {
@@ -1094,23 +1162,26 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
   }
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid), dim3(256), lds, stream, p);
+  hipLaunchKernelGGL(kernel, dim3((uint32_t)grid, (uint32_t)nproj), dim3(256), lds, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
+// Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
+// more of them resident hide more of each other's waits), four for a single projection (all of
+// its workgroups are resident at once, and four leave 128 registers: nothing spills).
 template <typename T, int NPROJ, bool PLANNED>
-__global__ __launch_bounds__(256, 5) void bgmv_expand_kernel(const ExpandArgs p) {
+__global__ __launch_bounds__(256, NPROJ == 3 ? 5 : 4) void bgmv_expand_kernel(const ExpandArgs p) {
   __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
-  expand_body<T, NPROJ, PLANNED>(p, (int)blockIdx.x, s_out[threadIdx.x >> 6]);
+  expand_body<T, NPROJ, PLANNED>(p, (int)blockIdx.x, (int)blockIdx.y, s_out[threadIdx.x >> 6]);
 }
 
 template <typename T, int NPROJ, bool PLANNED>
 int launch_expand(ExpandArgs p, int64_t items, hipStream_t stream) {
-  p.units = (int)items;
-  const int64_t grid = items * 2 * NPROJ;
+  const int64_t grid = items;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), dim3((uint32_t)grid), dim3(256), 0, stream, p);
+  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), dim3((uint32_t)grid, 2 * NPROJ), dim3(256), 0, stream,
+                     p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -1213,6 +1284,15 @@ int expand_prepare(const void* plan, int64_t n_items, int64_t rank_cap, void* co
     p.y[i] = i < nproj ? y[i] : nullptr;
     p.x[i] = i < nproj ? x[i] : nullptr;
     p.h_out[i] = i < nproj ? (int)h_out[i] : 0;
+    p.pages_shift[i] = -2;
+    if (i < nproj && h_out[i] > 0) {
+      if (h_out[i] >= page_elems) {
+        p.pages_shift[i] = -1;
+      } else if (page_elems % h_out[i] == 0) {
+        const int64_t q = page_elems / h_out[i];
+        if ((q & (q - 1)) == 0) p.pages_shift[i] = __builtin_ctzll((unsigned long long)q);
+      }
+    }
     if (i < nproj && h_out[i] > h_max) h_max = h_out[i];
   }
   if (h_max == 0) return kNothingToDo;

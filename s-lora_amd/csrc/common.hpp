@@ -35,6 +35,10 @@ struct F16 {
     _Float16 s = __builtin_bit_cast(_Float16, y) + __builtin_bit_cast(_Float16, d);
     return __builtin_bit_cast(uint16_t, s);
   }
+  // the same on both halves of a packed word (v_pk_add_f16)
+  static __device__ __forceinline__ uint32_t add2(uint32_t y, uint32_t d) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2, y) + __builtin_bit_cast(f16x2, d));
+  }
 };
 
 struct BF16 {
@@ -55,6 +59,10 @@ struct BF16 {
     // the sum of two bf16 values is exact in float unless their exponents are
     // more than 16 apart, where the smaller one cannot move the rounding
     return from_float(to_float(y) + to_float(d));
+  }
+  static __device__ __forceinline__ uint32_t add2(uint32_t y, uint32_t d) {
+    return (uint32_t)add((uint16_t)(y & 0xffffu), (uint16_t)(d & 0xffffu)) |
+           ((uint32_t)add((uint16_t)(y >> 16), (uint16_t)(d >> 16)) << 16);
   }
 };
 
