@@ -230,6 +230,26 @@ SLORA_API int slora_pool_scatter_rows(void* const* dst_bufs, const void* const* 
                             const int64_t* loc, int64_t n_rows, int64_t row_bytes, int64_t dst_row_stride_bytes,
                             int64_t src_row_stride_bytes, int64_t n_pages, void* stream);
 
+/* One adapter's LoRA matrices written straight into its pool pages, n_mats matrices per
+ * call (e.g. A_q, A_k, A_v, A_o into the key_buffer and B_q .. B_o into the value_buffer of
+ * every layer).  Replaces building w_combined on the host
+ * (slora/models/peft/layer_weights/lora_layer_weight.py:84-93, 215-224) and the index_put
+ * of its rows (slora/server/router/model_infer/infer_adapter.py:56-57, 81-82) with one pass.
+ * Matrix i is a (rows[i] x cols[i]) row-major device array of 16-bit elements -- A_p as the
+ * reference keeps it at home, (hidden x r), or B_p, (r x h_out).  It is written TRANSPOSED:
+ * element (k, c) goes to flat position c * dst_pitch[i] + k of the slot formed by the pages
+ * loc[first[i] .. first[i] + n_slot[i]) of dst_bufs[i], page flat / page_elems, offset flat
+ * % page_elems.  dst_pitch = page_elems for A_p (column j of A_p becomes page j), dst_pitch
+ * = rows = r for B_p (the dense (h_out, r) matrix B_p^T end to end); n_slot = r for both.
+ * Positions of the slot no source element reaches are zeroed (what index_put of the
+ * zero-padded w_combined leaves there).  first, rows, cols, dst_pitch, n_slot, dst_bufs and
+ * src_mats are HOST arrays of n_mats entries; loc is the device array of page ids (n_loc
+ * entries); a page id outside [0, n_pages) is skipped. */
+SLORA_API int slora_pool_pack_transposed(void* const* dst_bufs, const void* const* src_mats, const int64_t* first,
+                                         const int64_t* rows, const int64_t* cols, const int64_t* dst_pitch,
+                                         const int64_t* n_slot, int n_mats, const int64_t* loc, int64_t n_loc,
+                                         int64_t page_elems, int64_t n_pages, void* stream);
+
 /* new_a_loc[new_a_start[i] + k] = old_a_loc[old_a_start[i] + k], k < old_a_len[i],
  * i < n_adapters.  Replaces launch_var_len_copy_triton
  * (slora/server/router/model_infer/infer_adapter.py:261-280); copies exactly

@@ -111,6 +111,66 @@ __global__ __launch_bounds__(256) void pool_scatter_kernel(const ScatterArgs p) 
 }
 
 // ---------------------------------------------------------------------------
+// pack one adapter's matrices straight into its pool pages
+// ---------------------------------------------------------------------------
+// The adapter loader of the reference first builds w_combined on the host
+// (slora/models/peft/layer_weights/lora_layer_weight.py:84-93: A_p^T as r rows of hidden
+// elements, and the (h_out, r) row-major B_p^T cut into r rows) and then index_puts its rows
+// into the pool (infer_adapter.py:56-57, 81-82).  Both halves are the same operation: a
+// (rows x cols) row-major source matrix -- A_p is (hidden x r), B_p is (r x h_out) -- is
+// written transposed, as the (cols x rows) matrix whose rows are dst_pitch elements apart,
+// end to end over the pool pages loc[first .. first + n_slot): element (c, k) goes to flat
+// position c * dst_pitch + k, page flat / page_elems, offset flat % page_elems.  A_p uses
+// dst_pitch = page_elems (every column of A_p gets a page of its own), B_p uses dst_pitch =
+// rows (= r: dense).  Positions of the slot that no source element reaches are zeroed, as
+// index_put of the zero-padded w_combined would leave them.
+constexpr int kPackMats = 64;  // matrices per launch (their descriptions travel as kernel arguments)
+
+struct PackEntry {
+  void* dst;        // pool buffer
+  const void* src;  // (rows x cols) row-major, 16-bit elements
+  int64_t first;    // index of the slot's first page id in loc
+  int rows, cols, dst_pitch, n_slot;
+};
+struct PackArgs {
+  PackEntry m[kPackMats];
+  const int64_t* loc;
+  int64_t n_loc, n_pages, page_elems;
+  int n_mats, tiles_k;  // tiles_k: 64-wide tiles along k the grid provides per 64 columns
+};
+
+// 64 x 64 tiles through LDS: the source is read along its rows (cols contiguous), the
+// pages are written along k (contiguous).
+__global__ __launch_bounds__(256) void pool_pack_kernel(const PackArgs p) {
+  __shared__ uint16_t s_t[64][66];
+  const PackEntry e = p.m[blockIdx.y];
+  const int tile_c = (int)blockIdx.x / p.tiles_k, tile_k = (int)blockIdx.x - tile_c * p.tiles_k;
+  const int c0 = tile_c * 64, k0 = tile_k * 64;
+  const int64_t slot_elems = (int64_t)e.n_slot * p.page_elems;
+  if (k0 >= e.dst_pitch || (int64_t)c0 * e.dst_pitch >= slot_elems) return;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  const uint16_t* src = static_cast<const uint16_t*>(e.src);
+  for (int kk = ty; kk < 64; kk += 4) {
+    const int k = k0 + kk, c = c0 + tx;
+    s_t[kk][tx] = (k < e.rows && c < e.cols) ? src[(int64_t)k * e.cols + c] : (uint16_t)0;
+  }
+  __syncthreads();
+  uint16_t* dst = static_cast<uint16_t*>(e.dst);
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int c = c0 + cc, k = k0 + tx;
+    if (k >= e.dst_pitch) continue;
+    const int64_t flat = (int64_t)c * e.dst_pitch + k;
+    if (flat >= slot_elems) continue;
+    const int64_t pg = flat / p.page_elems, off = flat - pg * p.page_elems;
+    const int64_t li = e.first + pg;
+    if ((uint64_t)li >= (uint64_t)p.n_loc) continue;
+    const int64_t page = p.loc[li];
+    if ((uint64_t)page >= (uint64_t)p.n_pages) continue;  // a page id outside the pool is skipped
+    dst[page * p.page_elems + off] = s_t[tx][cc];
+  }
+}
+
+// ---------------------------------------------------------------------------
 // variable-length copy of page-id lists
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void var_len_copy_kernel(const int64_t* __restrict__ old_start,
@@ -518,6 +578,62 @@ int slora_pool_scatter_rows(void* const* dst_bufs, const void* const* src_bufs, 
     const int64_t grid = n_rows * p.n_bufs;
     if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(pool_scatter_kernel, dim3((uint32_t)grid), dim3(256), 0, s, p);
+    if (hipGetLastError() != hipSuccess) return SLORA_ERR_LAUNCH;
+  }
+  return SLORA_OK;
+}
+
+int slora_pool_pack_transposed(void* const* dst_bufs, const void* const* src_mats, const int64_t* first,
+                               const int64_t* rows, const int64_t* cols, const int64_t* dst_pitch,
+                               const int64_t* n_slot, int n_mats, const int64_t* loc, int64_t n_loc,
+                               int64_t page_elems, int64_t n_pages, void* stream) {
+  using namespace slora;
+  if (n_mats < 0 || n_loc < 0 || page_elems < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n_mats == 0) return SLORA_OK;
+  if (dst_bufs == nullptr || src_mats == nullptr || first == nullptr || rows == nullptr || cols == nullptr ||
+      dst_pitch == nullptr || n_slot == nullptr || loc == nullptr)
+    return SLORA_ERR_NULL_POINTER;
+  if (page_elems == 0) return SLORA_ERR_BAD_SHAPE;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  for (int m0 = 0; m0 < n_mats; m0 += kPackMats) {
+    PackArgs p{};
+    p.n_mats = n_mats - m0 < kPackMats ? n_mats - m0 : kPackMats;
+    int64_t max_tiles = 0;
+    int tiles_k = 1;
+    for (int i = 0; i < p.n_mats; ++i) {
+      const int j = m0 + i;
+      if (rows[j] < 0 || cols[j] < 0 || dst_pitch[j] < rows[j] || n_slot[j] < 0 || first[j] < 0)
+        return SLORA_ERR_BAD_SHAPE;
+      if (rows[j] > (1 << 24) || cols[j] > (1 << 24) || dst_pitch[j] > (1 << 30) || n_slot[j] > (1 << 20))
+        return SLORA_ERR_UNSUPPORTED;
+      // the transposed matrix must fit its slot
+      if (cols[j] > 0 && (cols[j] - 1) * dst_pitch[j] + rows[j] > n_slot[j] * page_elems) return SLORA_ERR_BAD_SHAPE;
+      if (dst_bufs[j] == nullptr || (src_mats[j] == nullptr && rows[j] * cols[j] > 0)) return SLORA_ERR_NULL_POINTER;
+      const int tk = (int)((dst_pitch[j] + 63) / 64);
+      if (tk > tiles_k) tiles_k = tk;
+    }
+    p.tiles_k = tiles_k;
+    for (int i = 0; i < p.n_mats; ++i) {
+      const int j = m0 + i;
+      p.m[i].dst = dst_bufs[j];
+      p.m[i].src = src_mats[j];
+      p.m[i].first = first[j];
+      p.m[i].rows = (int)rows[j];
+      p.m[i].cols = (int)cols[j];
+      p.m[i].dst_pitch = (int)dst_pitch[j];
+      p.m[i].n_slot = (int)n_slot[j];
+      // columns the slot has room for (source columns, then zero fill)
+      const int64_t c_cover = dst_pitch[j] > 0 ? (n_slot[j] * page_elems + dst_pitch[j] - 1) / dst_pitch[j] : 0;
+      const int64_t tiles = (c_cover + 63) / 64 * tiles_k;
+      if (tiles > max_tiles) max_tiles = tiles;
+    }
+    p.loc = loc;
+    p.n_loc = n_loc;
+    p.n_pages = n_pages;
+    p.page_elems = page_elems;
+    if (max_tiles == 0) continue;
+    if (max_tiles > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(pool_pack_kernel, dim3((uint32_t)max_tiles, (uint32_t)p.n_mats), dim3(256), 0, s, p);
     if (hipGetLastError() != hipSuccess) return SLORA_ERR_LAUNCH;
   }
   return SLORA_OK;

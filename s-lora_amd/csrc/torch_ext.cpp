@@ -727,6 +727,40 @@ void load_rows_into_pool(const std::vector<Tensor>& buffers, const std::vector<T
   for (const Tensor& b : buffers) mark_written(b);
 }
 
+// (rows x cols) matrices written transposed into the pool pages loc[first .. first + n_slot)
+void pack_transposed_into_pool(const std::vector<Tensor>& buffers, const std::vector<Tensor>& mats,
+                               const std::vector<int64_t>& first, const std::vector<int64_t>& dst_pitch,
+                               const std::vector<int64_t>& n_slot, const Tensor& loc) {
+  const size_t n = buffers.size();
+  TORCH_CHECK(mats.size() == n && first.size() == n && dst_pitch.size() == n && n_slot.size() == n,
+              "buffers, mats, first, dst_pitch and n_slot must have one entry per matrix");
+  if (n == 0) return;
+  SL_CHECK_INPUT(loc);
+  SL_CHECK_INDEX(loc);
+  const Tensor& b0 = buffers[0];
+  const int64_t page_elems = b0.size(0) > 0 ? b0.numel() / b0.size(0) : 0;
+  std::vector<void*> dst(n);
+  std::vector<const void*> src(n);
+  std::vector<int64_t> rows(n), cols(n);
+  for (size_t i = 0; i < n; ++i) {
+    const Tensor &b = buffers[i], &m = mats[i];
+    TORCH_CHECK(b.is_cuda() && b.is_contiguous(), "buffers[", i, "] must be a contiguous CUDA tensor");
+    TORCH_CHECK(m.is_cuda() && m.is_contiguous() && m.dim() == 2, "mats[", i, "] must be a contiguous 2D CUDA tensor");
+    TORCH_CHECK(b.element_size() == 2 && m.scalar_type() == b.scalar_type(),
+                "pool buffers and matrices must share one 16-bit dtype");
+    TORCH_CHECK(b.sizes() == b0.sizes(), "pool buffers must share one shape");
+    dst[i] = b.data_ptr();
+    src[i] = m.data_ptr();
+    rows[i] = m.size(0);
+    cols[i] = m.size(1);
+  }
+  const int rc = slora_pool_pack_transposed(dst.data(), src.data(), first.data(), rows.data(), cols.data(),
+                                            dst_pitch.data(), n_slot.data(), (int)n, loc.data_ptr<int64_t>(), loc.numel(),
+                                            page_elems, b0.size(0), stream_of(loc));
+  check_rc(rc, "pack_transposed_into_pool");
+  for (const Tensor& b : buffers) mark_written(b);
+}
+
 void launch_var_len_copy(const Tensor& old_a_start, const Tensor& old_a_len, const Tensor& old_location,
                          const Tensor& new_a_start, const Tensor& new_a_location) {
   for (const Tensor* t : {&old_a_start, &old_a_len, &old_location, &new_a_start, &new_a_location}) {
@@ -902,6 +936,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("b_seq_len"), py::arg("b_indicies"), py::arg("n_tokens"), py::arg("max_rank"), py::arg("max_input_len"));
 
   m.def("load_rows_into_pool", &load_rows_into_pool, py::arg("buffers"), py::arg("rows"), py::arg("loc"));
+  m.def("pack_transposed_into_pool", &pack_transposed_into_pool, py::arg("buffers"), py::arg("mats"), py::arg("first"),
+        py::arg("dst_pitch"), py::arg("n_slot"), py::arg("loc"));
   m.def("launch_var_len_copy", &launch_var_len_copy);
   m.def("compact_adapter_tables_raw", &compact_adapter_tables_raw);
   m.def("pool_alloc_workspace_bytes", &pool_alloc_workspace_bytes);

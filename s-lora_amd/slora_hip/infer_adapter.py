@@ -3,8 +3,16 @@ side of ``InferAdapter`` (slora/server/router/model_infer/infer_adapter.py).
 
 * ``load_rows_into_pool``    -- ``buffer[loc] = rows`` for many buffers in one launch
                                (``load_lora_A`` / ``load_lora_B``, :43-88).
+* ``pack_lora_into_pool``    -- A_p / B_p as the reference keeps them at home, transposed and
+                               written straight into the adapter's pages: ``w_combined``
+                               (slora/models/peft/layer_weights/lora_layer_weight.py:84-93)
+                               and its index_put in one pass.
 * ``launch_var_len_copy``    -- same arguments as ``launch_var_len_copy_triton`` (:274-280).
 * ``compact_adapter_tables`` -- the table rebuild of ``offload_adapters`` (:186-258).
+* ``InferAdapter``           -- the class itself: ``load_adapters`` / ``offload_adapters`` over
+                               the four index tables (:11-39, 92-258).
+* ``MemoryAllocator``        -- the reference's pool object (buffers + free map) on
+                               ``PageAllocator``, with a placement call for adapters.
 
 * ``PageAllocator``          -- ``MemoryAllocator.alloc / alloc_contiguous / free``
                                (slora/common/mem_allocator.py:30-59, 185-199) on the device.
@@ -16,6 +24,9 @@ side of ``InferAdapter`` (slora/server/router/model_infer/infer_adapter.py).
 All of them call libslora_hip.so through the compiled extension; there is no fallback.
 """
 from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List
 
 import torch
 
@@ -136,3 +147,226 @@ def unmerge_adapter(weights, key_buffer, value_buffer, a_start, a_len, a_loc, a_
     """``weights[p] -= scaling * A_p @ B_p`` (lora_single_batch_infer.py:78-93)."""
     merge_adapter(weights, key_buffer, value_buffer, a_start, a_len, a_loc, a_scaling, adapter_idx, sign=-1.0,
                   start=start, rank=rank)
+
+
+def pack_lora_into_pool(key_buffers, value_buffers, lora_A, lora_B, loc, rank: int) -> None:
+    """Write one adapter into its pool pages ``loc`` (``4 * rank`` page ids, the same in every
+    layer): ``lora_A[l][p]`` is A_p of layer l as the reference keeps it at home,
+    ``[hidden, rank]`` (``q_lora_A_home`` ... of lora_layer_weight.py:57-76, 170-213), and
+    ``lora_B[l][p]`` is B_p, ``[rank, h_out_p]``, p in q, k, v, o.  Page ``loc[p*rank + j]`` of
+    ``key_buffers[l]`` receives column j of A_p; the pages ``loc[p*rank ..]`` of
+    ``value_buffers[l]`` receive the ``(h_out_p, rank)`` row-major matrix B_p^T end to end
+    (lora_layer_weight.py:84-93): what ``w_combined`` holds, without building it.  One launch
+    per 8 layers."""
+    n_layers = len(key_buffers)
+    if not (len(value_buffers) == len(lora_A) == len(lora_B) == n_layers):
+        raise RuntimeError("key_buffers, value_buffers, lora_A and lora_B must have one entry per layer")
+    rank = int(rank)
+    if rank <= 0 or n_layers == 0:
+        return
+    page_elems = key_buffers[0][0].numel() if key_buffers[0].size(0) else 0
+    bufs, mats, first, pitch, slot = [], [], [], [], []
+    for l in range(n_layers):
+        if len(lora_A[l]) != 4 or len(lora_B[l]) != 4:
+            raise RuntimeError("every layer needs the q, k, v, o matrices")
+        for p in range(4):
+            a, b = lora_A[l][p], lora_B[l][p]
+            if a.dim() != 2 or a.size(1) != rank or b.dim() != 2 or b.size(0) != rank:
+                raise RuntimeError(f"layer {l} projection {p}: A must be [hidden, {rank}] and B [{rank}, h_out], got "
+                                   f"{tuple(a.shape)} and {tuple(b.shape)}")
+            bufs += [key_buffers[l], value_buffers[l]]
+            mats += [a, b]
+            first += [p * rank, p * rank]
+            pitch += [page_elems, rank]
+            slot += [rank, rank]
+    _kernels.pack_transposed_into_pool(bufs, mats, first, pitch, slot, loc)
+
+
+class MemoryAllocator(PageAllocator):
+    """``MemoryAllocator`` of slora/common/mem_allocator.py:10-234 with the same constructor,
+    attributes and calls: per-layer ``key_buffer`` / ``value_buffer`` of ``[tot_size, head_num,
+    head_dim]`` shared by the KV cache and the adapters, and the free map of ``PageAllocator``.
+
+    ``alloc_adapter`` is the placement call for adapter pages (not in the reference, whose
+    ``alloc`` hands out the first free pages wherever they lie, mem_allocator.py:30-39): one
+    contiguous run when the map has one, so that an adapter's ``4 r`` pages are one stretch of
+    the pool; the first free pages otherwise."""
+
+    def __init__(self, tot_size, cache_size, dtype, head_num, head_dim, layer_num, device="cuda"):
+        assert tot_size >= cache_size
+        self.dtype = dtype
+        self.head_num = head_num
+        self.head_dim = head_dim
+        self.layer_num = layer_num
+        self.cell_size = head_num * head_dim
+        self.cache_size = cache_size
+        super().__init__(tot_size, device)
+        self.key_buffer = [torch.empty((self.tot_size, head_num, head_dim), dtype=dtype, device=self.device)
+                           for _ in range(layer_num)]
+        self.value_buffer = [torch.empty((self.tot_size, head_num, head_dim), dtype=dtype, device=self.device)
+                             for _ in range(layer_num)]
+
+    def get_memory_size(self):
+        return 2 * self.layer_num * self.tot_size * self.cell_size * torch.empty((), dtype=self.dtype).element_size()
+
+    def alloc_adapter(self, need_size: int) -> torch.Tensor:
+        need_size = int(need_size)
+        if need_size <= 0:
+            return torch.empty(0, dtype=torch.int64, device=self.device)
+        got = self.alloc_contiguous(need_size)
+        return got[0] if got is not None else self.alloc(need_size)
+
+
+@dataclass
+class InferAdapter:
+    """The adapters that live in the pool and their index tables
+    (slora/server/router/model_infer/infer_adapter.py:11-258): adapter i owns the page ids
+    ``a_loc[a_start[i] : a_start[i] + a_len[i]]``, ``a_len[i] = 4 * rank``, ``a_scaling[i] =
+    lora_alpha / rank``.  Same fields and calls as the reference's class.
+
+    An adapter passed to ``load_adapters`` has ``lora_dir``, ``r``, ``scaling`` and either
+    ``layers`` whose entries offer ``load_to_gpu()`` / ``w_combined`` / ``offload_from_gpu()``
+    (the reference's ``LoraLayerWeight``: the rows are scattered into every layer's buffers in
+    one launch) or ``lora_A`` / ``lora_B`` (per layer the q, k, v, o matrices ``[hidden, r]`` /
+    ``[r, h_out]`` on the device: packed straight into the pages by ``pack_lora_into_pool``).
+    ``placement=True`` asks the pool for one contiguous run per adapter
+    (``MemoryAllocator.alloc_adapter``) instead of the reference's single ``alloc`` of the sum."""
+    adapter_dirs: List[str]
+    a_loc: torch.Tensor
+    a_start: torch.Tensor
+    a_len: torch.Tensor
+    a_scaling: torch.Tensor
+    mem_manager: Any
+    idx_map: Dict[str, int] = field(default_factory=dict)
+    prefetch_tag: Dict[str, int] = field(default_factory=dict)
+    cur_tag: int = 0
+    prefetch_stream: Any = None
+    placement: bool = False
+    len_host: List[int] = field(default_factory=list)   # a_len on the host, kept in step with the tables
+
+    @classmethod
+    def init(cls, mem_manager, prefetch_stream=None, placement=False, device="cuda"):
+        dev = torch.device(device)
+        return cls(adapter_dirs=[],
+                   a_loc=torch.empty(0, dtype=torch.long, device=dev),
+                   a_start=torch.empty(0, dtype=torch.long, device=dev),
+                   a_len=torch.empty(0, dtype=torch.long, device=dev),
+                   a_scaling=torch.empty(0, dtype=torch.float16, device=dev),
+                   mem_manager=mem_manager, idx_map={}, prefetch_tag={}, cur_tag=0,
+                   prefetch_stream=prefetch_stream, placement=placement)
+
+    # ---- one adapter's weights into the pages `loc` of every layer (load_lora_A + load_lora_B, :43-88)
+    def _load_weights(self, adapter, loc) -> None:
+        mm = self.mem_manager
+        if getattr(adapter, "lora_A", None) is not None:
+            pack_lora_into_pool(mm.key_buffer, mm.value_buffer, adapter.lora_A, adapter.lora_B, loc, adapter.r)
+            return
+        for layer in adapter.layers:
+            layer.load_to_gpu()
+        load_rows_into_pool(list(mm.key_buffer) + list(mm.value_buffer),
+                            [layer.w_combined[0] for layer in adapter.layers] +
+                            [layer.w_combined[1] for layer in adapter.layers], loc)
+        for layer in adapter.layers:
+            layer.offload_from_gpu()
+
+    def load_adapters(self, adapters, prefetch=False) -> None:
+        if len(adapters) == 0:
+            return
+        new_adapters, tot_size = [], 0
+        if prefetch:
+            self.cur_tag ^= 1
+            capacity = self.mem_manager.can_use_mem_size
+            for adapter in adapters:
+                if adapter is None:
+                    continue
+                self.prefetch_tag[adapter.lora_dir] = self.cur_tag
+                if adapter.lora_dir not in self.idx_map and adapter not in new_adapters:
+                    if tot_size + adapter.r * 4 > capacity:
+                        break
+                    new_adapters.append(adapter)
+                    tot_size += adapter.r * 4
+        else:
+            for adapter in adapters:
+                if adapter is not None and adapter.lora_dir not in self.idx_map and adapter not in new_adapters:
+                    new_adapters.append(adapter)
+                    tot_size += adapter.r * 4
+        if not new_adapters:
+            return
+        dev = self.a_loc.device
+        if self.placement and hasattr(self.mem_manager, "alloc_adapter"):
+            new_loc = torch.cat([self.mem_manager.alloc_adapter(a.r * 4) for a in new_adapters])
+        else:
+            new_loc = self.mem_manager.alloc(tot_size)
+        # the new adapters' tables, built on the host (sizes are host values) and appended in one go each
+        lens = [a.r * 4 for a in new_adapters]
+        starts, cum = [], 0
+        loc_offset = self.a_loc.shape[0]
+        for a, n in zip(new_adapters, lens):
+            starts.append(loc_offset + cum)
+            self.idx_map[a.lora_dir] = len(self.adapter_dirs)
+            self.adapter_dirs.append(a.lora_dir)
+            self.len_host.append(n)
+            cum += n
+        self.a_start = torch.cat((self.a_start, torch.tensor(starts, dtype=torch.long, device=dev)))
+        self.a_len = torch.cat((self.a_len, torch.tensor(lens, dtype=torch.long, device=dev)))
+        self.a_loc = torch.cat((self.a_loc, new_loc))
+        self.a_scaling = torch.cat((self.a_scaling, torch.tensor([a.scaling for a in new_adapters],
+                                                                 dtype=torch.float16, device=dev)))
+
+        def copy_all():
+            cum = 0
+            for a, n in zip(new_adapters, lens):
+                self._load_weights(a, new_loc[cum: cum + n])
+                cum += n
+
+        if prefetch and self.prefetch_stream is not None:
+            self.prefetch_stream.wait_stream(torch.cuda.current_stream())  # new_loc is produced on this stream
+            with torch.cuda.stream(self.prefetch_stream):
+                copy_all()
+        else:
+            copy_all()
+
+    def offload_adapters(self, reserve_adapter_dirs) -> None:
+        if len(reserve_adapter_dirs) == len(self.adapter_dirs):
+            return
+        dev = self.a_loc.device
+        if len(reserve_adapter_dirs) == 0:
+            self.mem_manager.free(self.a_loc)
+            self.adapter_dirs = []
+            self.a_loc = torch.empty(0, dtype=torch.long, device=dev)
+            self.a_start = torch.empty(0, dtype=torch.long, device=dev)
+            self.a_len = torch.empty(0, dtype=torch.long, device=dev)
+            self.a_scaling = torch.empty(0, dtype=torch.float16, device=dev)
+            self.idx_map = {}
+            self.len_host = []
+            return
+        keep, new_dirs, idx_map = [], [], {}
+        for d in self.adapter_dirs:
+            drop = d not in reserve_adapter_dirs and self.prefetch_tag.get(d) != self.cur_tag
+            keep.append(not drop)
+            if not drop:
+                idx_map[d] = len(new_dirs)
+                new_dirs.append(d)
+        if all(keep):
+            return
+        self.idx_map = idx_map
+        self.adapter_dirs = new_dirs
+        self.len_host = [n for n, k in zip(self.len_host, keep) if k]
+        # a_len[left_ind], cumsum, a_scaling[left_ind], var_len_copy and the cat of the removed lists, one launch
+        self.a_start, self.a_len, self.a_loc, self.a_scaling, remove_ind = compact_adapter_tables(
+            self.a_start, self.a_len, self.a_loc, self.a_scaling, torch.tensor(keep, dtype=torch.bool, device=dev))
+        self.mem_manager.free(remove_ind)
+
+    def start_and_rank(self, lora_dir: str):
+        """``(a_start[i], a_len[i] // 4)`` of a loaded adapter from the host copy of the tables
+        (no device read-back): what ``merge_adapter`` needs to find its pages."""
+        i = self.idx_map[lora_dir]
+        return sum(self.len_host[:i]), self.len_host[i] // 4
+
+    def merge_adapter(self, weights, layer_id: int, lora_dir: str, sign: float = 1.0) -> None:
+        """``weights[p] += sign * scaling * A_p B_p`` for the q, k, v, o matrices of one layer
+        (slora/models/peft/lora_single_batch_infer.py:60-93) from the adapter's pool pages."""
+        start, rank = self.start_and_rank(lora_dir)
+        merge_adapter(weights, self.mem_manager.key_buffer[layer_id], self.mem_manager.value_buffer[layer_id],
+                      self.a_start, self.a_len, self.a_loc, self.a_scaling, self.idx_map[lora_dir], sign=sign,
+                      start=start, rank=rank)

@@ -222,3 +222,202 @@ def test_pool_ops_reject_bad_arguments(gpu):
     with pytest.raises(RuntimeError):
         compact_adapter_tables(loc, loc, loc, torch.zeros(3, device=gpu, dtype=torch.float16),
                                torch.ones(2, device=gpu, dtype=torch.bool))
+
+
+# ---------------------------------------------------------------------------
+# the packer and the InferAdapter class
+# ---------------------------------------------------------------------------
+class _Adapter:
+    """What InferAdapter.load_adapters needs of an adapter: name, rank, scaling and per layer
+    the q, k, v, o matrices as the reference keeps them at home (A_p [hidden, r], B_p [r, h_out])."""
+
+    def __init__(self, name, r, alpha, lora_A, lora_B):
+        self.lora_dir, self.r, self.scaling = name, r, alpha / r
+        self.lora_A, self.lora_B = lora_A, lora_B
+
+
+class _RefStyleLayer:
+    """A layer object with the reference's interface (lora_layer_weight.py:226-246): w_combined
+    appears on load_to_gpu() and goes away on offload_from_gpu()."""
+
+    def __init__(self, w_combined_home):
+        self.home, self.w_combined = w_combined_home, None
+
+    def load_to_gpu(self, prefetch=False):
+        self.w_combined = self.home
+
+    def offload_from_gpu(self):
+        self.w_combined = None
+
+
+def _np_mats(rng, hidden, h_out, r, n_layers, dtype):
+    A = [[O.round_to(rng.standard_normal((hidden, r)).astype(np.float32) / 8, dtype) for _ in range(4)]
+         for _ in range(n_layers)]
+    B = [[O.round_to(rng.standard_normal((r, h_out[p])).astype(np.float32) / 4, dtype) for p in range(4)]
+         for _ in range(n_layers)]
+    return A, B
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,page_elems,h_out,rank,n_layers", [
+    (256, 256, [256] * 4, 16, 3),
+    (512, 512, [512, 64, 64, 512], 64, 2),      # grouped-query k/v: B^T fills part of its slot, zeros behind
+    (192, 256, [256, 128, 128, 192], 8, 9),     # rows shorter than a page, more matrices than one launch takes
+    (128, 128, [128] * 4, 12, 1),               # a rank that is no multiple of 8
+])
+def test_pack_lora_into_pool_equals_w_combined_index_put(gpu, dtype, hidden, page_elems, h_out, rank, n_layers):
+    """A_p / B_p transposed straight into the pool pages give bit for bit what the oracle's
+    ``pack_w_combined`` + ``load_into_pool`` (= the reference's host-side w_combined and its
+    per-layer index_put) leave there; other pages keep their bytes."""
+    from slora_hip.infer_adapter import pack_lora_into_pool
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rng = np.random.default_rng(hidden + rank)
+    n_pages = 4 * rank + 37
+    loc_np = rng.permutation(n_pages)[: 4 * rank].astype(np.int64)
+    A, B = _np_mats(rng, hidden, h_out, rank, n_layers, dtype)
+    g = torch.Generator(device=gpu)
+    g.manual_seed(3)
+    keys = [torch.randn((n_pages, 2, page_elems // 2), generator=g, device=gpu).to(tdt) for _ in range(n_layers)]
+    vals = [torch.randn((n_pages, 2, page_elems // 2), generator=g, device=gpu).to(tdt) for _ in range(n_layers)]
+    want_k = [k.float().cpu().numpy().reshape(n_pages, page_elems).copy() for k in keys]
+    want_v = [v.float().cpu().numpy().reshape(n_pages, page_elems).copy() for v in vals]
+    for l in range(n_layers):
+        O.load_into_pool(want_k[l], want_v[l], O.pack_w_combined(A[l], B[l], page_elems), loc_np)
+    dA = [[torch.from_numpy(a).to(gpu, tdt) for a in A[l]] for l in range(n_layers)]
+    dB = [[torch.from_numpy(b).to(gpu, tdt) for b in B[l]] for l in range(n_layers)]
+    pack_lora_into_pool(keys, vals, dA, dB, torch.from_numpy(loc_np).to(gpu), rank)
+    torch.cuda.synchronize()
+    for l in range(n_layers):
+        assert np.array_equal(keys[l].float().cpu().numpy().reshape(n_pages, page_elems), want_k[l]), l
+        assert np.array_equal(vals[l].float().cpu().numpy().reshape(n_pages, page_elems), want_v[l]), l
+
+
+@pytest.mark.parametrize("placement", [False, True])
+def test_infer_adapter_load_offload_and_decode(gpu, placement):
+    """InferAdapter over a MemoryAllocator: adapters arrive in three loads (device matrices, and
+    objects with the reference's w_combined interface), some are dropped, one comes back.  After
+    every step the four tables equal the oracle's (build_tables appended per load,
+    ref_offload_tables per offload) with the page ids the oracle's allocator hands out, and
+    dispatch_bgmv over the pool gives the dense LoRA of every loaded adapter."""
+    from slora_hip import dispatch_bgmv
+    from slora_hip.infer_adapter import InferAdapter, MemoryAllocator
+    H, L, heads = 256, 2, 4
+    rng = np.random.default_rng(5)
+    mm = MemoryAllocator(600, 0, torch.float16, heads, H // heads, L, device=gpu)
+    for b in mm.key_buffer + mm.value_buffer:
+        b.zero_()
+    # some KV pages are in use between the adapters' pages
+    kv = mm.alloc(50)
+    mm.free(kv[::2].contiguous())
+    state = mm.mem_state.cpu().numpy().astype(np.uint8)
+    ia = InferAdapter.init(mm, prefetch_stream=torch.cuda.Stream(), placement=placement, device=gpu)
+    ranks = {"a": 8, "b": 16, "c": 32, "d": 8, "e": 64}
+    mats, adapters = {}, {}
+    for name, r in ranks.items():
+        A, B = _np_mats(rng, H, [H] * 4, r, L, "f16")
+        mats[name] = (A, B)
+        if name in ("b", "d"):   # the reference's interface: per layer a w_combined [2, 4r, heads, head_dim]
+            layers = [_RefStyleLayer(torch.from_numpy(O.pack_w_combined(A[l], B[l], H)).to(gpu, torch.float16)
+                                     .view(2, 4 * r, heads, H // heads)) for l in range(L)]
+            ad = _Adapter(name, r, 16.0, None, None)
+            ad.layers = layers
+        else:
+            ad = _Adapter(name, r, 16.0, [[torch.from_numpy(a).to(gpu, torch.float16) for a in A[l]] for l in range(L)],
+                          [[torch.from_numpy(b).to(gpu, torch.float16) for b in B[l]] for l in range(L)])
+        adapters[name] = ad
+
+    tables = dict(start=np.zeros(0, np.int64), len=np.zeros(0, np.int64), loc=np.zeros(0, np.int64),
+                  scal=np.zeros(0, np.float32), dirs=[])
+
+    def oracle_load(names):
+        new = [n for n in names if n not in tables["dirs"]]
+        if placement:
+            locs = []
+            for n in new:
+                got = O.ref_alloc_contiguous(state, 4 * ranks[n])
+                locs.append(got[0] if got is not None else O.ref_alloc(state, 4 * ranks[n]))
+            new_loc = np.concatenate(locs)
+        else:
+            new_loc = O.ref_alloc(state, sum(4 * ranks[n] for n in new))
+        s, ln, lc = O.build_tables([ranks[n] for n in new], new_loc)
+        tables["start"] = np.concatenate([tables["start"], s + tables["loc"].size])
+        tables["len"] = np.concatenate([tables["len"], ln])
+        tables["loc"] = np.concatenate([tables["loc"], lc])
+        tables["scal"] = np.concatenate([tables["scal"], [16.0 / ranks[n] for n in new]]).astype(np.float32)
+        tables["dirs"] += new
+
+    def oracle_offload(reserve):
+        keep = np.array([d in reserve for d in tables["dirs"]])
+        s, ln, lc, sc, removed = O.ref_offload_tables(tables["start"], tables["len"], tables["loc"], tables["scal"], keep)
+        O.ref_free(state, removed)
+        tables.update(start=s, len=ln, loc=lc, scal=sc, dirs=[d for d, k in zip(tables["dirs"], keep) if k])
+
+    def check():
+        torch.cuda.synchronize()
+        assert ia.adapter_dirs == tables["dirs"]
+        assert np.array_equal(ia.a_start.cpu().numpy(), tables["start"])
+        assert np.array_equal(ia.a_len.cpu().numpy(), tables["len"])
+        assert np.array_equal(ia.a_loc.cpu().numpy(), tables["loc"])
+        assert np.array_equal(ia.a_scaling.float().cpu().numpy(), tables["scal"])
+        assert np.array_equal(mm.mem_state.cpu().numpy().astype(np.uint8), state)
+        assert mm.can_use_mem_size == int(state.sum())
+        for i, d in enumerate(ia.adapter_dirs):
+            assert ia.idx_map[d] == i
+            assert ia.start_and_rank(d) == (int(tables["start"][i]), ranks[d])
+        if not ia.adapter_dirs:
+            return
+        # one token per loaded adapter through the kernels, layer 1, every projection
+        n = len(ia.adapter_dirs)
+        x_np = O.round_to(rng.standard_normal((n, H)).astype(np.float32), "f16")
+        x = torch.from_numpy(x_np).to(gpu, torch.float16)
+        bins = torch.arange(n, dtype=torch.int64, device=gpu)
+        for p in range(4):
+            d = torch.zeros((n, 64), dtype=torch.float16, device=gpu)
+            dispatch_bgmv(d, x, mm.key_buffer[1], ia.a_start, ia.a_len, ia.a_loc, bins, p, ia.a_scaling)
+            y = torch.zeros((n, H), dtype=torch.float16, device=gpu)
+            dispatch_bgmv(y, d, mm.value_buffer[1], ia.a_start, ia.a_len, ia.a_loc, bins, p, ia.a_scaling)
+            want = np.stack([(x_np[i].astype(np.float64) @ mats[dn][0][1][p] @ mats[dn][1][1][p]) * 16.0 / ranks[dn]
+                             for i, dn in enumerate(ia.adapter_dirs)])
+            np.testing.assert_allclose(y.float().cpu().numpy(), want, rtol=2e-2, atol=2e-2)
+
+    ia.load_adapters([adapters["a"], adapters["b"]])
+    oracle_load(["a", "b"])
+    check()
+    ia.load_adapters([adapters["b"], adapters["c"], adapters["d"]], prefetch=True)   # b is there already
+    torch.cuda.current_stream().wait_stream(ia.prefetch_stream)
+    oracle_load(["c", "d"])
+    check()
+    ia.prefetch_tag.clear()                      # nothing is protected by a prefetch any more
+    ia.offload_adapters(["a", "c"])
+    oracle_offload(["a", "c"])
+    check()
+    ia.load_adapters([adapters["e"], adapters["b"]])
+    oracle_load(["e", "b"])
+    check()
+    ia.offload_adapters(["a", "c", "e", "b"])     # everything reserved: nothing happens
+    check()
+    ia.offload_adapters([])
+    oracle_offload([])
+    check()
+    assert mm.can_use_mem_size == 600 - 25
+
+
+def test_memory_allocator_places_an_adapter_in_one_run(gpu):
+    """alloc_adapter: one contiguous stretch when the map has one (the first such), the first
+    free pages otherwise -- against the oracle's alloc_contiguous / alloc."""
+    from slora_hip.infer_adapter import MemoryAllocator
+    mm = MemoryAllocator(300, 0, torch.float16, 2, 8, 1, device=gpu)
+    rng = np.random.default_rng(9)
+    busy = rng.permutation(300)[:120].astype(np.int64)
+    all_pages = mm.alloc(300)
+    keep_free = np.setdiff1d(np.arange(300), busy)
+    mm.free(torch.from_numpy(keep_free).to(gpu))
+    state = np.zeros(300, np.uint8)
+    state[keep_free] = 1
+    for need in (3, 7, 2, 40, 5):
+        got = mm.alloc_adapter(need).cpu().numpy()
+        run = O.ref_alloc_contiguous(state, need)
+        want = run[0] if run is not None else O.ref_alloc(state, need)
+        assert np.array_equal(got, want), need
+        assert np.array_equal(mm.mem_state.cpu().numpy().astype(np.uint8), state)
+    assert all_pages.numel() == 300
