@@ -34,7 +34,7 @@ TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81403867,  # 75112411 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 71000741,     # the q/k/v launch
     ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281674768,  # 155648888 read + 126025879 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16>"): 142878462,  # 140909310 read + 1969152 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 1>"): 142878462,  # 140909310 read + 1969152 written
 }
 
 
@@ -350,6 +350,7 @@ def measure_prefill(args, torch, device):
     x = [torch.randn((T, H), generator=g, device=device, dtype=torch.float32).to(w.dtype) for _ in range(L)]
     y = [torch.zeros((T, H), device=device, dtype=w.dtype) for _ in range(L)]
     d = torch.zeros((T, R), device=device, dtype=w.dtype)
+    d3 = [torch.zeros((T, R), device=device, dtype=w.dtype) for _ in range(3)]
     t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
 
     def plan():  # once per prefill step, as the automatic cache does for a caller that passes none
@@ -363,11 +364,28 @@ def measure_prefill(args, torch, device):
                 slora_hip.lora_get_qkvo_fwd_shrink(x[l], w.key_buffer[l].view(-1, H), d, *t, H, p, R, seg.max_len,
                                                    plan=pl)
 
+    def qkv_shrink_sweep():  # 4 launches per layer keep the per-launch arithmetic below the same
+        pl = plan()
+        for l in range(L):
+            for _ in range(4):
+                slora_hip.lora_get_qkvo_fwd_shrink_qkv(x[l], w.key_buffer[l].view(-1, H), *d3, *t, H, R, seg.max_len,
+                                                       plan=pl)
+
     def expand_sweep():
         for l in range(L):
             for p in range(4):
                 slora_hip.lora_get_qkvo_fwd_expand(d, w.value_buffer[l].view(-1, H), y[l], w.a_scaling, *t, H, p, R,
                                                    seg.max_len)
+
+    def step_fused():  # x read once for q, k and v: 6 launches per layer
+        pl = plan()
+        for l in range(L):
+            key, val = w.key_buffer[l].view(-1, H), w.value_buffer[l].view(-1, H)
+            slora_hip.lora_get_qkvo_fwd_shrink_qkv(x[l], key, *d3, *t, H, R, seg.max_len, plan=pl)
+            for p in range(3):
+                slora_hip.lora_get_qkvo_fwd_expand(d3[p], val, y[l], w.a_scaling, *t, H, p, R, seg.max_len)
+            slora_hip.lora_get_qkvo_fwd_shrink(x[l], key, d, *t, H, 3, R, seg.max_len, plan=pl)
+            slora_hip.lora_get_qkvo_fwd_expand(d, val, y[l], w.a_scaling, *t, H, 3, R, seg.max_len)
 
     def step():
         pl = plan()
@@ -382,18 +400,21 @@ def measure_prefill(args, torch, device):
     wrap = (lambda f: graphed(f, torch)) if use_graph else (lambda f: f)
     reps = max(5, args.steps)
     ms_step = time_region(wrap(step), reps, args.warmup, torch)
+    ms_step_fused = time_region(wrap(step_fused), reps, args.warmup, torch)
     kernels = {}
-    flops = seg.flops(w, H)
-    for label, sweep, kname, nbytes in (
-            ("shrink", shrink_sweep, "sgmm_shrink_planned_kernel<BF16>", seg.shrink_bytes(w)),
-            ("expand", expand_sweep, "sgmm_expand_walk_kernel<BF16, 2>", seg.expand_bytes(w, H))):
+    flops1 = seg.flops(w, H)
+    for label, sweep, kname, nbytes, flops in (
+            ("shrink", shrink_sweep, "sgmm_shrink_planned_kernel<BF16, 1>", seg.shrink_bytes(w), flops1),
+            ("qkv_shrink", qkv_shrink_sweep, "sgmm_shrink_planned_kernel<BF16, 3>",
+             3 * seg.shrink_bytes(w) - 2 * T * H * 2, 3 * flops1),
+            ("expand", expand_sweep, "sgmm_expand_walk_kernel<BF16, 2>", seg.expand_bytes(w, H), flops1)):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
         kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
                           "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                           "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                           "TFLOPs": round(flops / us / 1e6, 1),
                           "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
-    dom = max(kernels.values(), key=lambda k: k["us_per_launch"])
+    dom = max((k for n, k in kernels.items() if n != "qkv_shrink"), key=lambda k: k["us_per_launch"])
     out = {
         "metric": "LoRA prefill tokens/s + achieved HBM GB/s (% peak), C3 segmented shrink/expand",
         "value": round(T / (ms_step * 1e-3 / L), 1),
@@ -402,6 +423,7 @@ def measure_prefill(args, torch, device):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": w.name, "layers": L, "tokens": T, "requests": int(seg.lens_np.size),
                    "launch": args.launch, "launches_per_step": 8 * L + 1},
+        "ms_per_step_qkv_fused": round(ms_step_fused, 4),
         "roofline": {"kernel": dom["kernel"], "bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": dom["frac"], "traffic": TRAFFIC_BYTES.get(("c3", dom["kernel"])),
                      "algorithmic_bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"]},
@@ -641,6 +663,7 @@ def main():
         free_workload(w, bufs, torch)
         c3 = measure_prefill(argparse.Namespace(layers=2, steps=10, warmup=3, launch="graph"), torch, device)
         out["prefill_c3"] = {"tokens_per_s_per_layer": c3["value"], "ms_per_layer": round(c3["ms_per_step"] / 2, 4),
+                             "ms_per_layer_qkv_fused": round(c3["ms_per_step_qkv_fused"] / 2, 4),
                              "tokens": c3["config"]["tokens"], "dtype": "bf16", "kernels": c3["kernels"]}
     if other_modes:
         out["modes"] = other_modes

@@ -199,6 +199,19 @@ SLORA_API int slora_sgmm_shrink_planned(const void* plan, void* o, const void* x
                               int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages,
                               int qkvo, int dtype, void* stream);
 
+/* Prefill shrink of q, k and v in ONE launch.  The reference issues three shrink calls per
+ * layer with the same x (slora/models/peft/lora_unordered_batch_infer.py:334-347, 374-381,
+ * 400-407); here every 64-row tile of x is read once and multiplied with the weight rows of
+ * the three projections in turn.  o_q / o_k / o_v are three [n_tokens, >= max_rank] outputs
+ * with one row stride; per projection the results are those of slora_sgmm_shrink with qkvo =
+ * 0, 1, 2, bit for bit.  plan: NULL, or a plan of slora_sgmm_plan_build for this batch
+ * (SLORA_ERR_BAD_SHAPE if the batch shape takes no plan, as for slora_sgmm_shrink_planned). */
+SLORA_API int slora_sgmm_shrink_qkv(const void* plan, void* o_q, void* o_k, void* o_v, const void* x, const void* w,
+                          const slora_tables* tables, const int32_t* b_start_loc, const int32_t* b_seq_len,
+                          const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
+                          int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride,
+                          int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int dtype, void* stream);
+
 /* Prefill (segmented) expand.  Replaces lora_get_qkvo_fwd_expand + _expand_fwd_kernel
  * (lora_prefill.py:105-136, 10-54).
  *   o[row, n] = T( f32(o[row, n]) + (sum_{d < r_a} f32(x[row, d]) * f32(Bt[n*r_a + d])) * f32(scales[a]) )

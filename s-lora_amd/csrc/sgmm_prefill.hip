@@ -79,12 +79,13 @@ __device__ __forceinline__ bool seg_lookup(const SegTables& t, int req, int64_t&
 // shrink
 // ---------------------------------------------------------------------------
 struct SegShrinkArgs {
-  void* o;
+  void* o[3];  // one output per projection of the launch (q, k, v when nproj = 3)
   const void* x;
   const void* w;
   SegTables t;
   int64_t x_stride, w_stride, o_stride;  // elements per row
   int h_in, max_rank, qkvo, m_tiles;
+  int nproj;  // 1: projection qkvo; 3: q, k and v in one pass over x (qkvo = 0)
   int col_split;  // 1, 2 or 4 workgroups share a tile's rank columns (16-column tiles t with t % col_split == group)
   int vec_ok;  // every row start is 16-byte aligned and h_in % 8 == 0
 };
@@ -98,10 +99,10 @@ constexpr int kShrLd = kShrNB + 4;              // LDS row pitch (floats) -> con
 
 // Element-wise fallback for layouts the vector path cannot read.
 template <typename T>
-__device__ void shrink_generic(const SegShrinkArgs& p, int r_eff, int64_t base_li, int row0, int m0, int m_cnt) {
+__device__ void shrink_generic(const SegShrinkArgs& p, int pj, int r_eff, int64_t base_li, int row0, int m0, int m_cnt) {
   const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x);
   const uint16_t* w = reinterpret_cast<const uint16_t*>(p.w);
-  uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
+  uint16_t* o = reinterpret_cast<uint16_t*>(p.o[pj]);
   for (int idx = threadIdx.x; idx < m_cnt * p.max_rank; idx += kShrThreads) {
     const int m = idx / p.max_rank, j = idx - m * p.max_rank;
     const int64_t row = row0 + m0 + m;
@@ -201,19 +202,129 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
   if (i + 1 < n) mul_block(c1);
 }
 
+// The same share of the K loop for q, k and v at once: a 64-k block of the activations is
+// loaded once and multiplied with the block of each projection's weight rows in turn.  Two
+// activation blocks and two weight blocks are held; while one product runs, the weight block
+// it does not use is refilled with what is needed two products later (q, k, v of block i,
+// then q, k, v of block i + 1, ...), so every load has one product's time to arrive.  As in
+// shrink_k_loop no load sits inside a branch; loads past the last block re-read it.
+template <typename T, int NT, int MF>
+__device__ __forceinline__ void shrink_k_loop_qkv(const uint16_t* const (&xline)[kShrMF][2],
+                                                  const uint16_t* const (&wline)[3][4][2], int wave, int piece,
+                                                  int h_in, f32x4 (&acc)[3][kShrMF][4]) {
+  const int blocks = (h_in + 63) >> 6;
+  const int n = (blocks - wave + kShrWaves - 1) / kShrWaves;  // blocks of this wavefront
+  if (n <= 0) return;
+  const bool ragged_k = (h_in & 63) != 0;
+  struct ABlock {
+    u32x4 a[MF][2];
+  };
+  struct BBlock {
+    u32x4 b[NT][2];
+  };
+  auto k_of = [&](int i, bool& k_in) {
+    if (i >= n) i = n - 1;
+    int k = (i * kShrWaves + wave) * 64 + piece * 8;
+    k_in = k < h_in;
+    return k_in ? k : 0;
+  };
+  auto load_a = [&](int i, ABlock& blk) {
+    bool k_in;
+    const int k = k_of(i, k_in);
+#pragma unroll
+    for (int f = 0; f < MF; ++f)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16(xline[f][g] + k);
+    if (ragged_k && !k_in) {
+#pragma unroll
+      for (int f = 0; f < MF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();
+    }
+  };
+  auto load_b = [&](int i, int pj, BBlock& blk) {
+    bool k_in;
+    const int k = k_of(i, k_in);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) blk.b[t][g] = ldg16(wline[pj][t][g] + k);
+    if (ragged_k && !k_in) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) blk.b[t][0] = blk.b[t][1] = zero16();
+    }
+  };
+  auto to_mfma_order = [&](ABlock& blk) {
+#pragma unroll
+    for (int f = 0; f < MF; ++f) swap_halves(blk.a[f][0], blk.a[f][1]);
+  };
+  auto mul = [&](const ABlock& a, BBlock& b, f32x4 (&c)[kShrMF][4]) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) swap_halves(b.b[t][0], b.b[t][1]);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int f = 0; f < MF; ++f) c[f][t] = mfma16<T>(a.a[f][s], b.b[t][s], c[f][t]);
+  };
+  ABlock a0, a1;
+  BBlock bx, by;
+  load_a(0, a0);
+  load_b(0, 0, bx);
+  load_b(0, 1, by);
+  int i = 0;
+  // block i: activations in a0, q in bx, k in by
+  for (; i + 2 < n; i += 2) {
+    load_a(i + 1, a1);
+    to_mfma_order(a0);
+    mul(a0, bx, acc[0]);
+    load_b(i, 2, bx);
+    mul(a0, by, acc[1]);
+    load_b(i + 1, 0, by);
+    mul(a0, bx, acc[2]);
+    load_b(i + 1, 1, bx);
+    // block i + 1: activations in a1, q in by, k in bx
+    load_a(i + 2, a0);
+    to_mfma_order(a1);
+    mul(a1, by, acc[0]);
+    load_b(i + 1, 2, by);
+    mul(a1, bx, acc[1]);
+    load_b(i + 2, 0, bx);
+    mul(a1, by, acc[2]);
+    load_b(i + 2, 1, by);
+  }
+  // one or two blocks are left; block i is loaded as at the top of the loop
+  load_a(i + 1, a1);
+  to_mfma_order(a0);
+  mul(a0, bx, acc[0]);
+  load_b(i, 2, bx);
+  mul(a0, by, acc[1]);
+  load_b(i + 1, 0, by);
+  mul(a0, bx, acc[2]);
+  load_b(i + 1, 1, bx);
+  const bool second = i + 1 < n;
+  if (second) {
+    to_mfma_order(a1);
+    mul(a1, by, acc[0]);
+  }
+  load_b(i + 1, 2, by);
+  if (second) {
+    mul(a1, bx, acc[1]);
+    mul(a1, by, acc[2]);
+  }
+}
+
 // One tile: token rows row_first .. row_first + m_cnt (m_cnt <= kShrTM) of a request
 // whose weight rows start at a_loc[base_li]; of every 64 rank columns the 16-column
 // tiles t with t % p.col_split == cg.  All threads of the workgroup call it together;
 // it ends with a barrier.
-template <typename T>
+template <typename T, int NPROJ>
 __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_part, int64_t row_first, int m_cnt,
-                                            int r_eff, int64_t base_li, int cg) {
+                                            int r_eff, int64_t base_li, int rank, int cg) {
   const int cs = p.col_split;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
   const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
-  uint16_t* og = reinterpret_cast<uint16_t*>(p.o);
   const int lr = lane & 15, lg = lane >> 4;  // MFMA order: fragment row / k-group of this lane
   const int lrow = lr & 7, piece = lg + 4 * (lr >> 3);  // line order: row inside a half fragment, 16-byte piece
 
@@ -234,39 +345,56 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
     // this workgroup's tiles of the pass: cg, cg + cs, ...; n_own of them hold columns of the adapter
     const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
     const int n_own = n_tiles > cg ? (n_tiles - cg + cs - 1) / cs : 0;
+    f32x4 acc[NPROJ][kShrMF][4];
     if (n_own > 0) {
-      // weight rows of the lane's two loads per B fragment: the page lookups go out
-      // together; a row that does not exist (j >= r_eff, bad page id) reads pool page
-      // 0 -- its products only reach output columns that are zeroed below
-      const uint16_t* wline[4][2];
+      // weight rows of the lane's two loads per B fragment, for every projection of the
+      // launch (projection pj's rows start rank entries of a_loc behind the one before):
+      // the page lookups go out together; a row that does not exist (j >= r_eff, bad page
+      // id) reads pool page 0 -- its products only reach output columns that are zeroed below
+      const uint16_t* wline[NPROJ][4][2];
       {
-        int64_t pg[4][2];
+        int64_t pg[NPROJ][4][2];
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int pj = 0; pj < NPROJ; ++pj)
 #pragma unroll
-          for (int g = 0; g < 2; ++g) {
-            const int j = nb0 + (cg + cs * t) * 16 + 8 * g + lrow;
-            pg[t][g] = seg_page_nobranch(p.t, base_li + j, t < n_own && j < r_eff && p.t.n_loc > 0);
-          }
+          for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int g = 0; g < 2; ++g) {
+              const int j = nb0 + (cg + cs * t) * 16 + 8 * g + lrow;
+              pg[pj][t][g] = seg_page_nobranch(p.t, base_li + (int64_t)pj * rank + j,
+                                               t < n_own && j < r_eff && p.t.n_loc > 0);
+            }
 #pragma unroll
-          for (int g = 0; g < 2; ++g) wline[t][g] = wg + (pg[t][g] >= 0 ? pg[t][g] : 0) * p.w_stride;
+        for (int pj = 0; pj < NPROJ; ++pj)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int g = 0; g < 2; ++g) wline[pj][t][g] = wg + (pg[pj][t][g] >= 0 ? pg[pj][t][g] : 0) * p.w_stride;
       }
-      f32x4 acc[kShrMF][4];
 #pragma unroll
-      for (int f = 0; f < kShrMF; ++f)
+      for (int pj = 0; pj < NPROJ; ++pj)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int f = 0; f < kShrMF; ++f)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[pj][f][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
       // fragments that hold no row or no rank column are neither loaded nor multiplied
       auto k_loop = [&](auto mf) {
         constexpr int MF = decltype(mf)::value;
-        switch (n_own) {
-          case 1: shrink_k_loop<T, 1, MF>(xline, wline, wave, piece, p.h_in, acc); break;
-          case 2: shrink_k_loop<T, 2, MF>(xline, wline, wave, piece, p.h_in, acc); break;
-          case 3: shrink_k_loop<T, 3, MF>(xline, wline, wave, piece, p.h_in, acc); break;
-          default: shrink_k_loop<T, 4, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+        if constexpr (NPROJ == 1) {
+          switch (n_own) {
+            case 1: shrink_k_loop<T, 1, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+            case 2: shrink_k_loop<T, 2, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+            case 3: shrink_k_loop<T, 3, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+            default: shrink_k_loop<T, 4, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+          }
+        } else {
+          switch (n_own) {
+            case 1: shrink_k_loop_qkv<T, 1, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+            case 2: shrink_k_loop_qkv<T, 2, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+            case 3: shrink_k_loop_qkv<T, 3, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+            default: shrink_k_loop_qkv<T, 4, MF>(xline, wline, wave, piece, p.h_in, acc); break;
+          }
         }
       };
       switch ((m_cnt + 15) >> 4) {
@@ -275,31 +403,38 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
         case 3: k_loop(std::integral_constant<int, 3>{}); break;
         default: k_loop(std::integral_constant<int, 4>{}); break;
       }
-      // C tile: lane holds column lr, rows 4*lg + i; fragment t is column tile cg + cs * t
-      float* mine = s_part + wave * (kShrTM * kShrLd);
-#pragma unroll
-      for (int f = 0; f < kShrMF; ++f)
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-          if (t < n_own) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              mine[(f * 16 + lg * 4 + i) * kShrLd + (cg + cs * t) * 16 + lr] = acc[f][t][i];
-          }
     }
-    __syncthreads();
-    for (int idx = tid; idx < kShrTM * kShrNB; idx += kShrThreads) {
-      const int m = idx / kShrNB, c = idx - m * kShrNB;
-      if (m < m_cnt && c < nb_cnt && ((c >> 4) & (cs - 1)) == cg) {
-        float v = 0.f;
-        if (nb0 + c < r_eff) {
+    // the partial tiles of the four wavefronts are summed through LDS, one projection at a time
 #pragma unroll
-          for (int wv = 0; wv < kShrWaves; ++wv) v += s_part[wv * (kShrTM * kShrLd) + m * kShrLd + c];
-        }
-        og[(row_first + m) * p.o_stride + nb0 + c] = T::from_float(v);
+    for (int pj = 0; pj < NPROJ; ++pj) {
+      if (n_own > 0) {
+        // C tile: lane holds column lr, rows 4*lg + i; fragment t is column tile cg + cs * t
+        float* mine = s_part + wave * (kShrTM * kShrLd);
+#pragma unroll
+        for (int f = 0; f < kShrMF; ++f)
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (t < n_own) {
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                mine[(f * 16 + lg * 4 + i) * kShrLd + (cg + cs * t) * 16 + lr] = acc[pj][f][t][i];
+            }
       }
+      __syncthreads();
+      uint16_t* og = reinterpret_cast<uint16_t*>(p.o[pj]);
+      for (int idx = tid; idx < kShrTM * kShrNB; idx += kShrThreads) {
+        const int m = idx / kShrNB, c = idx - m * kShrNB;
+        if (m < m_cnt && c < nb_cnt && ((c >> 4) & (cs - 1)) == cg) {
+          float v = 0.f;
+          if (nb0 + c < r_eff) {
+#pragma unroll
+            for (int wv = 0; wv < kShrWaves; ++wv) v += s_part[wv * (kShrTM * kShrLd) + m * kShrLd + c];
+          }
+          og[(row_first + m) * p.o_stride + nb0 + c] = T::from_float(v);
+        }
+      }
+      __syncthreads();
     }
-    __syncthreads();
   }
 }
 
@@ -369,7 +504,7 @@ __device__ __forceinline__ int shrink_chunks_needed(int units, int r_eff, uint32
 // read the same weight rows, share an L2) and every workgroup the same cost,
 // whatever the mix of request lengths and ranks.  A workgroup owns the units
 // whose start falls into its part and walks them as tiles of up to kShrMF units.
-template <typename T>
+template <typename T, int NPROJ>
 __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   __shared__ int64_t s_wave[kShrWaves];
@@ -558,10 +693,12 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
         if (m_end > rows) m_end = rows;
         if (m_end <= m0) continue;
         if (!p.vec_ok) {
-          if (cg == 0) shrink_generic<T>(p, r_eff, base_li, rw0, m0, m_end - m0);
+          if (cg == 0)
+            for (int pj = 0; pj < NPROJ; ++pj)
+              shrink_generic<T>(p, pj, r_eff, base_li + (int64_t)pj * rj, rw0, m0, m_end - m0);
           __syncthreads();
         } else {
-          shrink_tile<T>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, cg);
+          shrink_tile<T, NPROJ>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, rj, cg);
         }
       }
     }
@@ -655,7 +792,7 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_plan_kernel(int* plan, SegTa
   }
 }
 
-template <typename T>
+template <typename T, int NPROJ>
 __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(const SegShrinkArgs p, const int* plan) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   const int slot = (int)(blockIdx.x & 7) * ((int)gridDim.x >> 3) + (int)(blockIdx.x >> 3);
@@ -673,10 +810,12 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(con
   for (int m0 = 0; m0 < m_rows; m0 += kShrTM) {
     const int m_cnt = m_rows - m0 < kShrTM ? m_rows - m0 : kShrTM;
     if (!p.vec_ok) {
-      if (cg == 0) shrink_generic<T>(p, r_eff, base_li, row_first, m0, m_cnt);
+      if (cg == 0)
+        for (int pj = 0; pj < NPROJ; ++pj)
+          shrink_generic<T>(p, pj, r_eff, base_li + (int64_t)pj * r, row_first, m0, m_cnt);
       __syncthreads();
     } else {
-      shrink_tile<T>(p, s_part, (int64_t)row_first + m0, m_cnt, r_eff, base_li, cg);
+      shrink_tile<T, NPROJ>(p, s_part, (int64_t)row_first + m0, m_cnt, r_eff, base_li, r, cg);
     }
   }
 }
@@ -1156,7 +1295,7 @@ bool shrink_plan_usable(int64_t n_requests, int64_t m_tiles, int64_t grid, int c
   return grid > 0 && n_requests <= kShrChunk && n_requests <= grid / cs && m_tiles <= 1024;
 }
 
-template <typename T>
+template <typename T, int NPROJ>
 int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t stream) {
   const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
   int64_t grid = 0;
@@ -1164,8 +1303,8 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
   shrink_geometry(p.t.n_tokens, p.t.n_requests, p.m_tiles, p.max_rank, grid, q.col_split);
   if (grid <= 0) return SLORA_OK;
   if (plan != nullptr && !shrink_plan_usable(p.t.n_requests, p.m_tiles, grid, q.col_split)) return SLORA_ERR_BAD_SHAPE;
-  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T>)
-                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T>);
+  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ>)
+                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ>);
   static bool attr_done[2] = {false, false};  // benign if two threads race: the call is idempotent
   if (!attr_done[plan != nullptr]) {
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
@@ -1175,9 +1314,10 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
     attr_done[plan != nullptr] = true;
   }
   if (plan != nullptr)
-    hipLaunchKernelGGL(sgmm_shrink_planned_kernel<T>, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q, plan);
+    hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q,
+                       plan);
   else
-    hipLaunchKernelGGL(sgmm_shrink_kernel<T>, dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
+    hipLaunchKernelGGL((sgmm_shrink_kernel<T, NPROJ>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -1216,25 +1356,29 @@ int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
   return launch_seg_expand_ks<T, 4>(p, grid, stream);
 }
 
-int seg_shrink_common(const int* plan, bool planned, void* o, const void* x, const void* w, const slora_tables* tables,
+int seg_shrink_common(const int* plan, bool planned, void* const o[3], int nproj, const void* x, const void* w,
+                      const slora_tables* tables,
                       const int32_t* b_start_loc, const int32_t* b_seq_len, const int64_t* b_indicies,
                       int64_t n_requests, int64_t max_input_len, int64_t n_tokens, int64_t h_in, int64_t max_rank,
                       int64_t x_row_stride, int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
                       int dtype, void* stream) {
   if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
   if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || h_in < 0 || max_rank < 0) return SLORA_ERR_BAD_SHAPE;
-  if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
+  if (qkvo < 0 || qkvo + nproj > 4) return SLORA_ERR_BAD_SHAPE;
   if (x_row_stride < h_in || w_row_stride < h_in || o_row_stride < max_rank) return SLORA_ERR_BAD_SHAPE;
   if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0) return SLORA_OK;
   SegShrinkArgs p{};
   int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
   if (rc != SLORA_OK) return rc;
   if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
-  if (o == nullptr || x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (x == nullptr || w == nullptr) return SLORA_ERR_NULL_POINTER;
+  for (int i = 0; i < nproj; ++i)
+    if (o[i] == nullptr) return SLORA_ERR_NULL_POINTER;
   if (h_in == 0 || h_in > (1 << 21) || max_rank > SLORA_MAX_RANK) return SLORA_ERR_UNSUPPORTED;
   if (planned && (reinterpret_cast<uintptr_t>(plan) & 15) != 0) return SLORA_ERR_ALIGNMENT;
   if (max_input_len > n_tokens) max_input_len = n_tokens;  // no request is longer than the batch
-  p.o = o;
+  for (int i = 0; i < 3; ++i) p.o[i] = i < nproj ? o[i] : nullptr;
+  p.nproj = nproj;
   p.x = x;
   p.w = w;
   p.x_stride = x_row_stride;
@@ -1247,7 +1391,9 @@ int seg_shrink_common(const int* plan, bool planned, void* o, const void* x, con
   p.col_split = 1;
   p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16>(p, plan, s) : launch_seg_shrink<BF16>(p, plan, s);
+  if (nproj == 3)
+    return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 3>(p, plan, s) : launch_seg_shrink<BF16, 3>(p, plan, s);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 1>(p, plan, s) : launch_seg_shrink<BF16, 1>(p, plan, s);
 }
 
 }  // namespace
@@ -1259,7 +1405,8 @@ int slora_sgmm_shrink(void* o, const void* x, const void* w, const slora_tables*
                       const int32_t* b_seq_len, const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len,
                       int64_t n_tokens, int64_t h_in, int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride,
                       int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype, void* stream) {
-  return slora::seg_shrink_common(nullptr, false, o, x, w, tables, b_start_loc, b_seq_len, b_indicies, n_requests,
+  void* const os[3] = {o, nullptr, nullptr};
+  return slora::seg_shrink_common(nullptr, false, os, 1, x, w, tables, b_start_loc, b_seq_len, b_indicies, n_requests,
                                   max_input_len, n_tokens, h_in, max_rank, x_row_stride, w_row_stride, o_row_stride,
                                   n_pages, qkvo, dtype, stream);
 }
@@ -1303,9 +1450,21 @@ int slora_sgmm_shrink_planned(const void* plan, void* o, const void* x, const vo
                               int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride, int64_t o_row_stride,
                               int64_t n_pages, int qkvo, int dtype, void* stream) {
   if (plan == nullptr) return SLORA_ERR_NULL_POINTER;
-  return slora::seg_shrink_common(static_cast<const int*>(plan), true, o, x, w, tables, b_start_loc, b_seq_len,
+  void* const os[3] = {o, nullptr, nullptr};
+  return slora::seg_shrink_common(static_cast<const int*>(plan), true, os, 1, x, w, tables, b_start_loc, b_seq_len,
                                   b_indicies, n_requests, max_input_len, n_tokens, h_in, max_rank, x_row_stride,
                                   w_row_stride, o_row_stride, n_pages, qkvo, dtype, stream);
+}
+
+int slora_sgmm_shrink_qkv(const void* plan, void* o_q, void* o_k, void* o_v, const void* x, const void* w,
+                          const slora_tables* tables, const int32_t* b_start_loc, const int32_t* b_seq_len,
+                          const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len, int64_t n_tokens,
+                          int64_t h_in, int64_t max_rank, int64_t x_row_stride, int64_t w_row_stride,
+                          int64_t o_row_stride, int64_t n_pages, int dtype, void* stream) {
+  void* const os[3] = {o_q, o_k, o_v};
+  return slora::seg_shrink_common(static_cast<const int*>(plan), plan != nullptr, os, 3, x, w, tables, b_start_loc,
+                                  b_seq_len, b_indicies, n_requests, max_input_len, n_tokens, h_in, max_rank,
+                                  x_row_stride, w_row_stride, o_row_stride, n_pages, 0, dtype, stream);
 }
 
 int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables* tables, const void* scales,

@@ -675,6 +675,36 @@ void lora_get_qkvo_fwd_shrink(const Tensor& x, const Tensor& w, const Tensor& o,
                  " qkvo=" + std::to_string(qkvo) + ")");
 }
 
+// q, k and v shrink of one layer in one pass over x (no counterpart in the reference, which
+// issues the three calls of lora_unordered_batch_infer.py:334-347, 374-381, 400-407)
+void lora_get_qkvo_fwd_shrink_qkv(const Tensor& x, const Tensor& w, const Tensor& o_q, const Tensor& o_k,
+                                  const Tensor& o_v, const Tensor& b_loc, const Tensor& b_lora_start,
+                                  const Tensor& b_lora_ranks, const Tensor& b_start_loc, const Tensor& b_seq_len,
+                                  const Tensor& b_indicies, int64_t hidden_size, int64_t max_rank,
+                                  int64_t max_input_len, const py::object& plan) {
+  const slora_tables t = prefill_common(x, w, o_q, b_loc, b_lora_start, b_lora_ranks, b_start_loc, b_seq_len, b_indicies);
+  check_2d_strided(o_k, "o_k");
+  check_2d_strided(o_v, "o_v");
+  TORCH_CHECK(o_k.scalar_type() == o_q.scalar_type() && o_v.scalar_type() == o_q.scalar_type() &&
+                  o_k.sizes() == o_q.sizes() && o_v.sizes() == o_q.sizes() && o_k.stride(0) == o_q.stride(0) &&
+                  o_v.stride(0) == o_q.stride(0),
+              "o_q, o_k and o_v must share dtype, shape and row stride");
+  TORCH_CHECK(x.size(1) >= hidden_size && w.size(1) >= hidden_size && o_q.size(1) >= max_rank,
+              "x/w narrower than hidden_size or o narrower than max_rank");
+  void* stream = stream_of(x);
+  const std::shared_ptr<SgmmPlan> p =
+      resolve_prefill_plan(plan, b_lora_start, b_lora_ranks, b_start_loc, b_seq_len, b_indicies, x.size(0), max_rank,
+                           max_input_len, stream, "lora_get_qkvo_fwd_shrink_qkv");
+  const int rc = slora_sgmm_shrink_qkv(p ? p->buf.data_ptr() : nullptr, o_q.data_ptr(), o_k.data_ptr(), o_v.data_ptr(),
+                                       x.data_ptr(), w.data_ptr(), &t, b_start_loc.data_ptr<int32_t>(),
+                                       b_seq_len.data_ptr<int32_t>(), b_indicies.data_ptr<int64_t>(), b_seq_len.numel(),
+                                       max_input_len, x.size(0), hidden_size, max_rank, x.stride(0), w.stride(0),
+                                       o_q.stride(0), w.size(0), dtype_code(x, "x"), stream);
+  if (rc != SLORA_OK)
+    check_rc(rc, "lora_get_qkvo_fwd_shrink_qkv",
+             "(hidden_size=" + std::to_string(hidden_size) + " max_rank=" + std::to_string(max_rank) + ")");
+}
+
 void lora_get_qkvo_fwd_expand(const Tensor& x, const Tensor& w, const Tensor& o, const Tensor& scale, const Tensor& b_loc,
                               const Tensor& b_lora_start, const Tensor& b_lora_ranks, const Tensor& b_start_loc,
                               const Tensor& b_seq_len, const Tensor& b_indicies, int64_t feat_out, int64_t qkvo,
@@ -929,6 +959,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("b_lora_start"), py::arg("b_lora_ranks"), py::arg("b_start_loc"), py::arg("b_seq_len"),
         py::arg("b_indicies"), py::arg("hidden_size"), py::arg("qkvo"), py::arg("max_rank"), py::arg("max_input_len"),
         py::arg("plan") = py::none());
+  m.def("lora_get_qkvo_fwd_shrink_qkv", &lora_get_qkvo_fwd_shrink_qkv, py::arg("x"), py::arg("w"), py::arg("o_q"),
+        py::arg("o_k"), py::arg("o_v"), py::arg("b_loc"), py::arg("b_lora_start"), py::arg("b_lora_ranks"),
+        py::arg("b_start_loc"), py::arg("b_seq_len"), py::arg("b_indicies"), py::arg("hidden_size"), py::arg("max_rank"),
+        py::arg("max_input_len"), py::arg("plan") = py::none());
   m.def("lora_get_qkvo_fwd_expand", &lora_get_qkvo_fwd_expand, py::arg("x"), py::arg("w"), py::arg("o"), py::arg("scale"),
         py::arg("b_loc"), py::arg("b_lora_start"), py::arg("b_lora_ranks"), py::arg("b_start_loc"), py::arg("b_seq_len"),
         py::arg("b_indicies"), py::arg("feat_out"), py::arg("qkvo"), py::arg("max_rank"), py::arg("max_input_len"));

@@ -17,4 +17,4 @@ last call with the same five index tensors is reused; ``plan=False`` forces the
 kernel that needs no plan.
 """
 from ._kernels import (SgmmPlan, clear_prefill_plan_cache, lora_get_qkvo_fwd_expand,  # noqa: F401
-                       lora_get_qkvo_fwd_shrink, make_prefill_plan)
+                       lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv, make_prefill_plan)

@@ -51,6 +51,8 @@ SIGNATURES = {
     "slora_sgmm_plan_build": (_I, [_P, _I64, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, C.POINTER(C.c_int), _P]),
     "slora_sgmm_shrink_planned": (_I, [_P, _P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                        _I64, _I, _I, _P]),
+    "slora_sgmm_shrink_qkv": (_I, [_P, _P, _P, _P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
+                                   _I64, _I64, _I, _P]),
     "slora_sgmm_expand": (_I, [_P, _P, _P, _TP, _P, _I, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I64, _I64, _I, _I, _P]),
     "slora_pool_scatter_rows": (_I, [_P, _P, _I, _P, _I64, _I64, _I64, _I64, _I64, _P]),

@@ -355,3 +355,57 @@ def test_prefill_plan_of_another_batch_is_rejected(gpu):
     with pytest.raises(RuntimeError, match="another batch"):
         lora_get_qkvo_fwd_shrink(g.x, g.key.view(c.n_pages, c.page_elems), o, g.a_loc, g.a_start, g.a_len, start, lens,
                                  ids, c.hidden, 0, 32, max_len, plan=plan)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,ranks,n_req,lo,hi,sort", [
+    (256, [8, 16, 32, 64], 9, 1, 70, True),        # small batch: rank columns shared by 4 workgroups
+    (1024, [64, 8, 16], 40, 30, 200, True),        # a few chunks per request
+    (4096, [64, 32, 16, 8], 12, 8, 300, True),     # the hidden size of the headline configurations
+    (320, [128, 24], 5, 1, 300, False),            # two passes over the rank; rank 24 takes the element-wise path
+    (256, [16, 32], 300, 1, 9, False),             # more requests than a plan describes
+    (200, [8, 40, 16], 7, 1, 90, False),           # hidden size that is no multiple of 64: ragged last k block
+    (64, [8], 3, 1, 20, True),                     # a single k block per row
+    (128, [16, 8], 4, 1, 30, True),                # two k blocks: fewer blocks than wavefronts
+])
+def test_prefill_qkv_shrink_gives_the_three_calls_bits(gpu, dtype, hidden, ranks, n_req, lo, hi, sort):
+    """lora_get_qkvo_fwd_shrink_qkv (x read once for q, k and v) against the three calls
+    the reference issues (lora_unordered_batch_infer.py:334-347 and the k, v blocks after
+    it): identical bits, with a plan and without; rows of no request and the columns
+    beyond max_rank stay as they were."""
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv
+    c = seg_case(1200 + hidden + n_req, hidden, ranks, n_req, lo, hi, dtype, sort=sort)
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    R = (max(ranks) + 7) // 8 * 8
+    w_a = g.key.view(c.n_pages, c.page_elems)
+    T = c.batch
+    x = torch.cat([g.x, torch.ones((3, c.hidden), dtype=g.tdt, device=gpu)])     # 3 rows owned by no request
+    t = (g.a_loc, g.a_start, g.a_len, start, lens, ids)
+    single = []
+    for p in range(3):
+        o = torch.full((T + 3, R + 8), 7.0, dtype=g.tdt, device=gpu)
+        lora_get_qkvo_fwd_shrink(x, w_a, o[:, :R], *t, c.hidden, p, R, max_len, plan=False)
+        single.append(o)
+    for how in (False, None):
+        fused = [torch.full((T + 3, R + 8), 7.0, dtype=g.tdt, device=gpu) for _ in range(3)]
+        lora_get_qkvo_fwd_shrink_qkv(x, w_a, fused[0][:, :R], fused[1][:, :R], fused[2][:, :R], *t, c.hidden, R, max_len,
+                                     plan=how)
+        torch.cuda.synchronize()
+        for p in range(3):
+            assert torch.equal(fused[p], single[p]), (p, how)
+    d_ref = O.ref_prefill_shrink(np.zeros((T, R), np.float32), c.x, c.key, c.a_loc, c.a_start, c.a_len, c.start,
+                                 c.lens, c.ids, 1, R, c.dtype)
+    np.testing.assert_allclose(host(single[1][:T, :R]), d_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_prefill_qkv_shrink_rejects_mismatched_outputs(gpu):
+    from slora_hip import lora_get_qkvo_fwd_shrink_qkv
+    c = seg_case(33, 256, [16, 8], 6, 1, 50, "f16")
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    o = [torch.zeros((c.batch, 16), dtype=g.tdt, device=gpu) for _ in range(2)]
+    wide = torch.zeros((c.batch, 24), dtype=g.tdt, device=gpu)
+    with pytest.raises(RuntimeError, match="share dtype, shape and row stride"):
+        lora_get_qkvo_fwd_shrink_qkv(g.x, g.key.view(c.n_pages, c.page_elems), o[0], o[1], wide, g.a_loc, g.a_start,
+                                     g.a_len, start, lens, ids, c.hidden, 16, max_len)
