@@ -321,7 +321,32 @@ def measure_dropin_direct(w, bufs, torch, args):
             slora_hip.dispatch_bgmv(d1, x1, w.key_buffer[0], *t, one, 0, w.a_scaling)
 
     host_us = wall_ms(calls, 3, 1)  # ms per 1000 calls = us per call
-    return {"dropin-direct-autoplan": {
+
+    # the same step through the engine class: one object per step (as model_rpc.py:234 builds it),
+    # q/k/v in one shrink and one expand launch, o as two calls
+    from types import SimpleNamespace
+    dirs = [f"adapter-{i}" for i in range(len(w.ranks))]
+    ia = SimpleNamespace(a_start=w.a_start, a_len=w.a_len, a_loc=w.a_loc, a_scaling=w.a_scaling, adapter_dirs=dirs,
+                         idx_map={d: i for i, d in enumerate(dirs)},
+                         mem_manager=SimpleNamespace(key_buffer=w.key_buffer, value_buffer=w.value_buffer))
+    reqs = [SimpleNamespace(lora_dir=dirs[a], r=int(w.ranks[a])) for a in w.bins_np]
+    b_start = torch.zeros(w.batch, dtype=torch.int32, device=w.req_bins.device)
+    b_len = torch.full((w.batch,), 100, dtype=torch.int32, device=w.req_bins.device)
+
+    def engine_step():
+        eng = slora_hip.LoraUnorderedBatchInfer(ia, reqs, fused=True)
+        eng.begin_step(b_start, b_len, is_prefill=False, max_b_seq_len=100)
+        for l in range(L):
+            eng.lora_get_qkv(l, bufs.x_in[l], bufs.y[l][0], bufs.y[l][1], bufs.y[l][2])
+            eng.lora_get_o(l, bufs.x_att[l], bufs.y[l][3])
+
+    ms_eng = wall_ms(engine_step, max(5, args.steps // 2), 3)
+    return {"engine-fused-direct": {
+        "what": "LoraUnorderedBatchInfer(fused=True) built anew every step: q/k/v in one shrink and one expand "
+                "launch per layer, direct launches from Python, plan built and reused by the library",
+        "ms_per_step": round(ms_eng, 4), "tokens_per_s": round(w.batch / (ms_eng * 1e-3), 1),
+        "launches_per_step": 4 * L + 2},
+        "dropin-direct-autoplan": {
         "what": "reference call pattern (8 dispatch_bgmv per layer, new req_bins per step), direct launches from "
                 "Python through the extension, plan built and reused by the library",
         "ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1), "launches_per_step": 8 * L + 2,
