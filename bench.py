@@ -57,6 +57,9 @@ def parse_args():
     ap.add_argument("--all-modes", action="store_true", help="also time the other modes and report them under 'modes'")
     ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
                     help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
+    ap.add_argument("--placement", choices=["scattered", "runs"], default="scattered",
+                    help="where the adapters' pages lie in the pool -- scattered (the metric's configuration) "
+                         "or one contiguous run per adapter (what MemoryAllocator.alloc_adapter asks for)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="leave out the 'modes' (reference call pattern, direct launches) and 'prefill_c3' blocks "
@@ -582,11 +585,13 @@ def main():
         main_load(args, torch, device)
         return
     if args.workload == "s2":
-        w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch)
+        w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch, placement=args.placement)
     elif args.workload == "s4":
-        w = workloads.s4_decode(device, n_layers=args.layers, batch=args.batch if args.batch != 256 else 512)
+        w = workloads.s4_decode(device, n_layers=args.layers, batch=args.batch if args.batch != 256 else 512,
+                                placement=args.placement)
     else:
-        w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024)
+        w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024,
+                                placement=args.placement)
     bufs = StepBuffers(w, device)
     step, families = make_step(w, bufs, args.mode)
     fused = args.mode.endswith("fused")
@@ -657,7 +662,7 @@ def main():
             "layers": w.n_layers,
             "batch": w.batch,
             "distinct_adapters_in_batch": int(w.distinct_adapters().size),
-            "pool_pages_per_layer": w.n_pages,
+            "pool_pages_per_layer": w.n_pages, "placement": args.placement,
             "mode": args.mode,
             "launch": args.launch,
             "launches_per_step": w.n_layers * (4 if fused else 8) +

@@ -163,7 +163,7 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
 #pragma unroll
     for (int f = 0; f < MF; ++f)
 #pragma unroll
-      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16(xline[f][g] + k);
+      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16_stream(xline[f][g] + k);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -234,7 +234,7 @@ __device__ __forceinline__ void shrink_k_loop_qkv(const uint16_t* const (&xline)
 #pragma unroll
     for (int f = 0; f < MF; ++f)
 #pragma unroll
-      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16(xline[f][g] + k);
+      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16_stream(xline[f][g] + k);
     if (ragged_k && !k_in) {
 #pragma unroll
       for (int f = 0; f < MF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();

@@ -104,8 +104,13 @@ def zipf_ids(rng, n_adapters: int, batch: int, alpha: float) -> np.ndarray:
 
 def build_decode_workload(name, device, *, hidden, n_layers, n_adapters, rank_choices, batch, n_pages,
                           dtype=torch.float16, h_out=None, ids="zipf", zipf_alpha=1.0, occupancy=0.6, heads=32,
-                          lora_alpha=16.0, seed=2, fill_noise=True) -> DecodeWorkload:
+                          lora_alpha=16.0, seed=2, fill_noise=True, placement="scattered") -> DecodeWorkload:
     """Allocate and fill the pools on ``device``.
+
+    ``placement``: "scattered" -- every adapter page at a random place of the pool (what an
+    allocator that hands out the first free pages of a fragmented map ends up with);
+    "runs" -- each adapter's ``4 r`` pages one contiguous run at a random place (what
+    ``MemoryAllocator.alloc_adapter`` asks for).
 
     Weights: A ~ N(0, 1/hidden), B ~ N(0, 1/r), scaling = lora_alpha / r; pages
     not owned by an adapter up to ``occupancy`` of the pool hold N(0,1) noise
@@ -123,9 +128,22 @@ def build_decode_workload(name, device, *, hidden, n_layers, n_adapters, rank_ch
     if n_loc > n_pages:
         raise ValueError(f"pool of {n_pages} pages cannot hold {n_loc} adapter pages")
     perm = rng.permutation(n_pages).astype(np.int64)
-    a_loc = perm[:n_loc]
     n_kv = max(0, int(occupancy * n_pages) - n_loc)
-    kv_pages = perm[n_loc:n_loc + n_kv]
+    if placement == "scattered":
+        a_loc = perm[:n_loc]
+        kv_pages = perm[n_loc:n_loc + n_kv]
+    elif placement == "runs":
+        # the pool cut into slots of the largest adapter's size; adapters take random slots
+        slot = int(a_len.max())
+        slots = rng.permutation(n_pages // slot)[:n_adapters].astype(np.int64)
+        if slots.size < n_adapters:
+            raise ValueError(f"pool of {n_pages} pages has no room for {n_adapters} runs of {slot} pages")
+        a_loc = np.concatenate([s0 * slot + np.arange(n, dtype=np.int64) for s0, n in zip(slots, a_len)])
+        used = np.zeros(n_pages, dtype=bool)
+        used[a_loc] = True
+        kv_pages = perm[~used[perm]][:n_kv]
+    else:
+        raise ValueError(f"unknown placement {placement!r}")
     scales = (lora_alpha / ranks).astype(np.float32)
     h_out = list(h_out) if h_out is not None else [hidden] * 4
     w = DecodeWorkload(name=name, hidden=hidden, h_out=h_out, n_layers=n_layers, ranks=ranks, bins_np=bins,
@@ -164,25 +182,28 @@ def build_decode_workload(name, device, *, hidden, n_layers, n_adapters, rank_ch
 
 # The benchmark configurations (hidden sizes and rank mixes of the S2 / S4 / S6
 # dummy setups).
-def s2_decode(device, n_layers=32, batch=256, n_pages=65536, dtype=torch.float16, seed=2):
+def s2_decode(device, n_layers=32, batch=256, n_pages=65536, dtype=torch.float16, seed=2, placement="scattered"):
     return build_decode_workload("S2 decode BGMV: hidden 4096, ranks {64,32,16,8}, 200 adapters, Zipf(1), batch 256",
                                  device, hidden=4096, n_layers=n_layers, n_adapters=200, rank_choices=[64, 32, 16, 8],
-                                 batch=batch, n_pages=n_pages, dtype=dtype, ids="zipf", zipf_alpha=1.0, seed=seed)
+                                 batch=batch, n_pages=n_pages, dtype=dtype, ids="zipf", zipf_alpha=1.0, seed=seed,
+                                 placement=placement)
 
 
-def s4_decode(device, n_layers=40, batch=512, n_pages=262144, dtype=torch.float16, seed=4):
+def s4_decode(device, n_layers=40, batch=512, n_pages=262144, dtype=torch.float16, seed=4, placement="scattered"):
     return build_decode_workload("S4 decode: hidden 5120, ranks {64,32,16}, 1000 adapters, Zipf(0.9), batch 512",
                                  device, hidden=5120, n_layers=n_layers, n_adapters=1000, rank_choices=[64, 32, 16],
                                  batch=batch, n_pages=n_pages, dtype=dtype, ids="zipf", zipf_alpha=0.9, heads=40,
-                                 seed=seed)
+                                 seed=seed, placement=placement)
 
 
-def s6_decode(device, n_layers=8, batch=1024, n_adapters=2000, n_pages=None, dtype=torch.bfloat16, seed=6):
+def s6_decode(device, n_layers=8, batch=1024, n_adapters=2000, n_pages=None, dtype=torch.bfloat16, seed=6,
+              placement="scattered"):
     n_pages = n_pages or (n_adapters * 256 + 4096)
     return build_decode_workload("S6 decode: hidden 8192, rank 64, 2000 adapters, uniform ids, batch 1024, GQA k/v 1024",
                                  device, hidden=8192, n_layers=n_layers, n_adapters=n_adapters, rank_choices=[64],
                                  batch=batch, n_pages=n_pages, dtype=dtype, h_out=[8192, 1024, 1024, 8192],
-                                 ids="uniform", heads=64, seed=seed, occupancy=0.0, fill_noise=False)
+                                 ids="uniform", heads=64, seed=seed, occupancy=0.0, fill_noise=False,
+                                 placement=placement)
 
 
 # ---- prefill ------------------------------------------------------------------
