@@ -642,6 +642,31 @@ def main():
                           "bytes_per_launch": int(nbytes), "GBps": round(gbs, 1),
                           "frac": round(gbs / HBM_PEAK_GBS, 4)}
     dom = max(kernels.values(), key=lambda k: k["us_per_launch"] * k["launches_per_step"])
+    if fused:
+        # streaming ceiling of each kind of launch: a checksum kernel (one wavefront per page, loads only)
+        # over exactly the weight pages that launch reads -- no activations, no outputs, no dependent lookups
+        import numpy as np
+        from slora_hip.infer_adapter import page_checksums
+        u = w.distinct_adapters()
+
+        def pages_of(projs):
+            idx = [w.a_start_np[a] + p * w.ranks[a] + np.arange(w.ranks[a]) for p in projs for a in u]
+            return torch.from_numpy(w.a_loc_np[np.concatenate(idx)]).to(device)
+
+        for label, projs, side in (("qkv_shrink", (0, 1, 2), w.key_buffer), ("o_shrink", (3,), w.key_buffer),
+                                   ("qkv_expand", (0, 1, 2), w.value_buffer), ("o_expand", (3,), w.value_buffer)):
+            loc = pages_of(projs)
+
+            def sweep(loc=loc, side=side):
+                for l in range(w.n_layers):
+                    page_checksums(side[l], loc)
+
+            fn = graphed(sweep, torch) if use_graph else sweep
+            us = time_region(fn, reps, 3, torch) * 1e3 / w.n_layers
+            nb = int(loc.numel()) * w.page_elems * 2
+            kernels[label]["read_only_ceiling"] = {"us": round(us, 3), "page_bytes": nb,
+                                                   "GBps": round(nb / us / 1e3, 1),
+                                                   "kernel_over_ceiling": round(kernels[label]["us_per_launch"] / us, 3)}
 
     step_gbs = w.step_bytes(fused) / (ms_per_step * 1e-3) / 1e9
     out = {

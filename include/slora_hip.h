@@ -300,6 +300,15 @@ SLORA_API int slora_tables_compact(const slora_tables* tables, const void* a_sca
 SLORA_API int slora_pool_gather_a(void* out, int64_t out_cols, const void* pool, const int64_t* a_loc, int64_t n_loc,
                         int64_t first, int64_t rank, int64_t h, int64_t page_elems, int64_t n_pages, void* stream);
 
+/* Checksums of pool pages: out[i] = xor of the 32-bit words of page loc[i] of `pool` (pages of
+ * page_bytes bytes, a multiple of 16; an id outside [0, n_pages) gives 0).  No counterpart in
+ * the reference, which has no way to tell whether the pages an adapter was copied into
+ * (slora/server/router/model_infer/infer_adapter.py:43-88) still hold it.  The kernel is one
+ * wavefront per page and only reads: the benchmark times it over the pages a LoRA launch
+ * reads and reports that as the streaming ceiling of the launch. */
+SLORA_API int slora_pool_page_checksums(uint32_t* out, const void* pool, const int64_t* loc, int64_t n,
+                                        int64_t page_bytes, int64_t n_pages, void* stream);
+
 /* ---- page allocator over the pool's free map ---------------------------------
  * mem_state: one byte per pool page, 1 = free (the reference's torch.bool
  * `mem_state`, slora/common/mem_allocator.py:222).  `workspace` is device memory of

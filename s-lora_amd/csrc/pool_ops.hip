@@ -329,6 +329,38 @@ __global__ __launch_bounds__(256) void gather_a_kernel(const uint16_t* __restric
 }
 
 // ---------------------------------------------------------------------------
+// checksum of pool pages: out[i] = xor of the 32-bit words of page loc[i].  One wavefront
+// per page, 16-byte loads, nothing else: the plainest read of scattered pages there is,
+// which makes its duration the streaming ceiling the LoRA kernels are measured against.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void page_xor_kernel(const u32x4* __restrict__ pool, int64_t page_vecs,
+                                                       int64_t n_pages, const int64_t* __restrict__ loc, int64_t n,
+                                                       uint32_t* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int64_t page = loc[i];
+  u32x4 acc = zero16();
+  if ((uint64_t)page < (uint64_t)n_pages) {
+    const u32x4* src = pool + page * page_vecs;
+    for (int64_t v0 = 0; v0 < page_vecs; v0 += 8 * kWave) {
+      u32x4 v[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const int64_t k = v0 + c * kWave + lane;
+        v[c] = k < page_vecs ? ldg16_stream(src + k) : zero16();
+      }
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc ^= v[c];
+    }
+  }
+  uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) r ^= (uint32_t)__shfl_xor((int)r, o, kWave);
+  if (lane == 0) out[i] = r;
+}
+
+// ---------------------------------------------------------------------------
 // page allocator over the free map (1 byte per page, 1 = free)
 // ---------------------------------------------------------------------------
 constexpr int kMapThreads = 256;
@@ -702,6 +734,21 @@ int slora_pool_gather_a(void* out, int64_t out_cols, const void* pool, const int
   hipLaunchKernelGGL(gather_a_kernel, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                      static_cast<const uint16_t*>(pool), page_elems, n_pages, a_loc, n_loc, first, (int)rank, (int)h,
                      static_cast<uint16_t*>(out), (int)out_cols);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_page_checksums(uint32_t* out, const void* pool, const int64_t* loc, int64_t n, int64_t page_bytes,
+                              int64_t n_pages, void* stream) {
+  using namespace slora;
+  if (n < 0 || page_bytes < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n == 0) return SLORA_OK;
+  if (out == nullptr || pool == nullptr || loc == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (page_bytes % 16 != 0) return SLORA_ERR_UNSUPPORTED;
+  if (!aligned16(pool)) return SLORA_ERR_ALIGNMENT;
+  const int64_t grid = (n + 3) / 4;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(page_xor_kernel, dim3((uint32_t)grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     static_cast<const u32x4*>(pool), page_bytes / 16, n_pages, loc, n, out);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 

@@ -888,6 +888,21 @@ void pool_free(const Tensor& mem_state, const Tensor& free_index) {
   mark_written(mem_state);
 }
 
+// xor of the 32-bit words of every listed pool page (int32 tensor, one entry per page)
+Tensor page_checksums(const Tensor& buffer, const Tensor& loc) {
+  SL_CHECK_INPUT(buffer);
+  SL_CHECK_INPUT(loc);
+  SL_CHECK_INDEX(loc);
+  TORCH_CHECK(buffer.dim() >= 1, "buffer must be [pages, ...]");
+  const int64_t n_pages = buffer.size(0);
+  const int64_t page_bytes = n_pages > 0 ? buffer.numel() / n_pages * buffer.element_size() : 0;
+  Tensor out = at::empty({loc.numel()}, loc.options().dtype(at::kInt));
+  const int rc = slora_pool_page_checksums(reinterpret_cast<uint32_t*>(out.data_ptr<int32_t>()), buffer.data_ptr(),
+                                           loc.data_ptr<int64_t>(), loc.numel(), page_bytes, n_pages, stream_of(buffer));
+  check_rc(rc, "page_checksums");
+  return out;
+}
+
 Tensor gather_lora_a(const Tensor& key_buffer, const Tensor& a_loc, int64_t first, int64_t rank, int64_t hidden,
                      int64_t out_cols) {
   SL_CHECK_INPUT(key_buffer);
@@ -979,6 +994,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("pool_alloc_contiguous", &pool_alloc_contiguous, py::arg("mem_state"), py::arg("need"), py::arg("out_index"),
         py::arg("result"), py::arg("work") = py::none());
   m.def("pool_free", &pool_free);
+  m.def("page_checksums", &page_checksums, py::arg("buffer"), py::arg("loc"));
   m.def("gather_lora_a", &gather_lora_a, py::arg("key_buffer"), py::arg("a_loc"), py::arg("first"), py::arg("rank"),
         py::arg("hidden"), py::arg("out_cols") = 0);
 }

@@ -94,6 +94,13 @@ class PageAllocator:
         self.can_use_mem_size = self.tot_size
 
 
+def page_checksums(buffer: torch.Tensor, loc: torch.Tensor) -> torch.Tensor:
+    """xor of the 32-bit words of each pool page ``buffer[loc[i]]`` (int32 tensor): a cheap way to
+    tell whether the pages an adapter was loaded into still hold what was written there.  A page id
+    outside the buffer gives 0."""
+    return _kernels.page_checksums(buffer, loc)
+
+
 def gather_lora_a(key_buffer, a_loc, first: int, rank: int, hidden: int, out_cols: int = 0) -> torch.Tensor:
     """``A_p`` as a dense ``[hidden, out_cols]`` tensor out of the pool pages
     ``a_loc[first : first + rank]`` (lora_single_batch_infer.py:38-46); columns

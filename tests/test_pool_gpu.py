@@ -421,3 +421,23 @@ def test_memory_allocator_places_an_adapter_in_one_run(gpu):
         assert np.array_equal(got, want), need
         assert np.array_equal(mm.mem_state.cpu().numpy().astype(np.uint8), state)
     assert all_pages.numel() == 300
+
+
+@pytest.mark.parametrize("dtype,heads,head_dim", [(torch.float16, 32, 128), (torch.bfloat16, 4, 24)])
+def test_page_checksums_equal_numpy_xor(gpu, dtype, heads, head_dim):
+    """page_checksums against the xor of the pages' 32-bit words computed with numpy: exact;
+    page ids outside the buffer give 0; an empty list gives an empty result."""
+    from slora_hip.infer_adapter import page_checksums
+    g = torch.Generator(device=gpu)
+    g.manual_seed(9)
+    buf = torch.randn((300, heads, head_dim), generator=g, device=gpu, dtype=torch.float32).to(dtype)
+    rng = np.random.default_rng(9)
+    loc = rng.integers(0, 300, size=1001).astype(np.int64)
+    loc[5], loc[77] = -1, 300
+    got = page_checksums(buf, torch.from_numpy(loc).to(gpu)).cpu().numpy().view(np.uint32)
+    words = buf.cpu().view(torch.int16).numpy().reshape(300, -1).view(np.uint32)
+    want = np.bitwise_xor.reduce(words, axis=1)
+    ok = (loc >= 0) & (loc < 300)
+    assert np.array_equal(got[ok], want[loc[ok]])
+    assert np.all(got[~ok] == 0)
+    assert page_checksums(buf, torch.empty(0, dtype=torch.int64, device=gpu)).numel() == 0
