@@ -649,13 +649,16 @@ def main():
         from slora_hip.infer_adapter import page_checksums
         u = w.distinct_adapters()
 
-        def pages_of(projs):
-            idx = [w.a_start_np[a] + p * w.ranks[a] + np.arange(w.ranks[a]) for p in projs for a in u]
+        def pages_of(projs, expand):
+            # A side: one page per rank row; B side: the r * h_out elements of B^T from the slot's first page on
+            def n_pages(a, p):
+                return -(-int(w.ranks[a]) * w.h_out[p] // w.page_elems) if expand else int(w.ranks[a])
+            idx = [w.a_start_np[a] + p * w.ranks[a] + np.arange(n_pages(a, p)) for p in projs for a in u]
             return torch.from_numpy(w.a_loc_np[np.concatenate(idx)]).to(device)
 
         for label, projs, side in (("qkv_shrink", (0, 1, 2), w.key_buffer), ("o_shrink", (3,), w.key_buffer),
                                    ("qkv_expand", (0, 1, 2), w.value_buffer), ("o_expand", (3,), w.value_buffer)):
-            loc = pages_of(projs)
+            loc = pages_of(projs, label.endswith("expand"))
 
             def sweep(loc=loc, side=side):
                 for l in range(w.n_layers):
