@@ -214,38 +214,40 @@ struct ShrinkArgs {
   int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
 };
 
-// The common case in straight-line code: hidden <= 4096 (one pass), all tokens
-// of the run fit the LDS staging area, no rows beyond the item.  Every global
-// load is unconditional (absent tokens / rows read a valid dummy address and are
-// discarded) so that no branch separates the loads: first the activations, then
+// The common case in straight-line code: the whole page in one pass (hidden <= 512 * NV
+// elements), all tokens of the run fit the LDS staging area, no rows beyond the item.
+// Every global load is unconditional (absent tokens / rows read a valid dummy address
+// and are discarded) so that no branch separates the loads: first the activations, then
 // both weight pages; the LDS stores wait for the activations only.
-template <typename T>
+// NV: 16-byte vectors a lane holds of a page (8 = hidden up to 4096).
+template <typename T, int NV>
 __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it, int proj, int r_eff,
                                             const int64_t (&page)[2], u32x4* s_x) {
+  constexpr int XS = (NV + 3) / 4;  // activation vectors a thread stages per token
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nvec = p.h_in >> 3;
   const u32x4* xg = reinterpret_cast<const u32x4*>(p.x);
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
 
-  u32x4 xr[kTT][2];
+  u32x4 xr[kTT][XS];
 #pragma unroll
   for (int t = 0; t < kTT; ++t) {
     const int tk = t < it.n_tok ? it.tok[t] : it.tok[0];
     const u32x4* xrow = xg + (int64_t)tk * nvec;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < XS; ++i) {
       const int v = i * 256 + tid;
       xr[t][i] = xrow[v < nvec ? v : 0];
     }
   }
   __builtin_amdgcn_sched_barrier(0);  // keep the activation loads in front: the LDS stores wait for them only
-  u32x4 wv[2][kVecPerPass];
+  u32x4 wv[2][NV];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const u32x4* src = reinterpret_cast<const u32x4*>(wbase + (page[i] >= 0 ? page[i] : 0) * p.page_elems);
 #pragma unroll
-    for (int c = 0; c < kVecPerPass; ++c) {
+    for (int c = 0; c < NV; ++c) {
       const int v = c * kWave + lane;
       wv[i][c] = ldg16_stream(src + (v < nvec ? v : 0));
     }
@@ -254,7 +256,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 #pragma unroll
   for (int t = 0; t < kTT; ++t)
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < XS; ++i) {
       const int v = i * 256 + tid;
       if (t < it.n_tok && v < nvec) s_x[t * nvec + v] = xr[t][i];
     }
@@ -269,7 +271,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
   for (int t = 0; t < kTT; ++t) {
     if (t < it.n_tok) {
 #pragma unroll
-      for (int c = 0; c < kVecPerPass; ++c) {
+      for (int c = 0; c < NV; ++c) {
         const int v = c * kWave + lane;
         if (v < nvec) {
           const u32x4 xv = s_x[t * nvec + v];
@@ -301,7 +303,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 // and share its activations in that L2).
 // Grid: x = item (planned) or token * blocks + block (stateless), y = projection of the
 // launch.  s_x: [lds_tt][h_in / 8] LDS words.
-template <typename T, bool PLANNED>
+template <typename T, bool PLANNED, int NV>
 __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int proj, u32x4* s_x) {
   constexpr int NW = 4;
   constexpr int NTASK = 2;
@@ -336,11 +338,11 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
   if (it.j0 >= r_eff) return;  // uniform over the workgroup
 
   const int nvec = p.h_in >> 3;
-  if (nvec <= 512 && it.n_tok <= p.lds_tt && !(PLANNED && it.more)) {
+  if (nvec <= NV * kWave && it.n_tok <= p.lds_tt && !(PLANNED && it.more)) {
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       if (it.j0 + wave + 4 * i >= r_eff) page2[i] = -1;
-    shrink_fast<T>(p, it, proj, r_eff, page2, s_x);
+    shrink_fast<T, NV>(p, it, proj, r_eff, page2, s_x);
     return;
   }
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
@@ -455,10 +457,12 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
   }
 }
 
-template <typename T, bool PLANNED>
+// NV: the straight-line path of this instantiation holds pages of up to 512 * NV elements
+// (8: hidden <= 4096; larger ones cost registers, so the host picks the smallest that fits)
+template <typename T, bool PLANNED, int NV>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];  // [lds_tt][h_in / 8]
-  shrink_body<T, PLANNED>(p, (int)blockIdx.x, (int)blockIdx.y, s_x);
+  shrink_body<T, PLANNED, NV>(p, (int)blockIdx.x, (int)blockIdx.y, s_x);
 }
 
 // ---------------------------------------------------------------------------
@@ -1142,16 +1146,9 @@ int64_t plan_words(int64_t batch, int64_t rank_cap) {
   return kPlanHeaderWords + plan_max_items(batch, rank_cap) * kItemWords + plan_scratch_words(batch);
 }
 
-template <typename T, bool PLANNED>
-int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
-  // as many tokens staged at once as fit a modest LDS budget
-  const size_t row_bytes = (size_t)p.h_in * 2;
-  int tt = kTT;
-  while (tt > 1 && tt * row_bytes > 32 * 1024) --tt;
-  const size_t lds = tt * row_bytes;
-  if (lds > kLdsHardLimit) return SLORA_ERR_UNSUPPORTED;
-  p.lds_tt = tt;
-  auto kernel = bgmv_shrink_kernel<T, PLANNED>;
+template <typename T, bool PLANNED, int NV>
+int launch_shrink_nv(ShrinkArgs p, int nproj, int64_t units, size_t lds, hipStream_t stream) {
+  auto kernel = bgmv_shrink_kernel<T, PLANNED, NV>;
   const int64_t grid = units;
   if (lds > kLdsSoftLimit) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1166,6 +1163,27 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
+template <typename T, bool PLANNED>
+int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
+  // as many tokens staged at once as fit the LDS budget: a full run of kTT tokens up to
+  // hidden 8192 (four workgroups per compute unit at 5120, two at 8192), fewer beyond
+  const size_t row_bytes = (size_t)p.h_in * 2;
+  int tt = kTT;
+  while (tt > 1 && tt * row_bytes > 64 * 1024) --tt;
+  const size_t lds = tt * row_bytes;
+  if (lds > kLdsHardLimit) return SLORA_ERR_UNSUPPORTED;
+  p.lds_tt = tt;
+  const int nvec = p.h_in >> 3;
+  if (nvec <= 8 * kWave) return launch_shrink_nv<T, PLANNED, 8>(p, nproj, units, lds, stream);
+  if (nvec <= 10 * kWave) return launch_shrink_nv<T, PLANNED, 10>(p, nproj, units, lds, stream);
+  if (nvec <= 12 * kWave) return launch_shrink_nv<T, PLANNED, 12>(p, nproj, units, lds, stream);
+  if (nvec <= 16 * kWave) return launch_shrink_nv<T, PLANNED, 16>(p, nproj, units, lds, stream);
+  return launch_shrink_nv<T, PLANNED, 8>(p, nproj, units, lds, stream);  // general path only
+}
+
+// Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
+// more of them resident hide more of each other's waits), four for a single projection (all of
+// its workgroups are resident at once, and four leave 128 registers: nothing spills).
 // Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
 // more of them resident hide more of each other's waits), four for a single projection (all of
 // its workgroups are resident at once, and four leave 128 registers: nothing spills).
