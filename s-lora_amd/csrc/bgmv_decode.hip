@@ -478,6 +478,8 @@ struct ExpandArgs {
   int64_t page_elems;
   int scales_dtype;
   int batch, x_cols, qkvo0, blocks, y_aligned;
+  int interleave;  // one-dimensional grid: the workgroups of an item follow each other (see bgmv_expand_kernel)
+  int n_units;     // items (planned) or token blocks (stateless) of the launch
   int h_out[3];
   // pages per rank row of each projection: a rank-r adapter's B^T fills ceil(r * h_out /
   // page_elems) pages.  pages_shift >= 0: page_elems = h_out << pages_shift (the count is a
@@ -1187,19 +1189,38 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
 // Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
 // more of them resident hide more of each other's waits), four for a single projection (all of
 // its workgroups are resident at once, and four leave 128 registers: nothing spills).
+// Grid, two forms.  Two-dimensional (x = unit, y = projection * 2 + half): all workgroups of
+// one projection half run before those of the next.  One-dimensional (p.interleave): id L
+// -> unit 8 * (L / (8 * S)) + L % 8, sub (L / 8) % S with S = 2 * NPROJ, so a unit still sits
+// on XCD unit % 8 and its S workgroups follow each other.  The second form is for outputs
+// narrower than a page (grouped-query k and v): most of their workgroups find no page and
+// exit, and spread between the others they cost nothing, while in phases of their own they
+// are all a phase consists of.
 template <typename T, int NPROJ, bool PLANNED>
 __global__ __launch_bounds__(256, NPROJ == 3 ? 5 : 4) void bgmv_expand_kernel(const ExpandArgs p) {
   __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
-  expand_body<T, NPROJ, PLANNED>(p, (int)blockIdx.x, (int)blockIdx.y, s_out[threadIdx.x >> 6]);
+  int unit = (int)blockIdx.x, sub = (int)blockIdx.y;
+  if (p.interleave) {
+    constexpr int S = 2 * NPROJ;
+    const int g = unit >> 3;
+    unit = (g / S) * 8 + (unit & 7);
+    sub = g % S;
+    if (unit >= p.n_units) return;
+  }
+  expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
 }
 
 template <typename T, int NPROJ, bool PLANNED>
 int launch_expand(ExpandArgs p, int64_t items, hipStream_t stream) {
-  const int64_t grid = items;
-  if (grid <= 0) return SLORA_OK;
-  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), dim3((uint32_t)grid, 2 * NPROJ), dim3(256), 0, stream,
-                     p);
+  if (items <= 0) return SLORA_OK;
+  if (items > 0x7fffffffLL / (2 * NPROJ + 1)) return SLORA_ERR_UNSUPPORTED;
+  p.n_units = (int)items;
+  p.interleave = 0;
+  for (int i = 0; i < NPROJ; ++i)
+    if (p.pages_shift[i] > 0) p.interleave = 1;  // an output narrower than a page
+  dim3 grid((uint32_t)items, 2 * NPROJ);
+  if (p.interleave) grid = dim3((uint32_t)((items + 7) / 8 * 8 * 2 * NPROJ), 1);
+  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), grid, dim3(256), 0, stream, p);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
