@@ -64,6 +64,20 @@ def run_chain(c, g, p, R, device, y0=None):
     return host(delta), host(y)
 
 
+def assert_close_but_for_rounding_flips(got, want, rtol, atol, dtype):
+    """rtol / atol as stated, except that at most 2 in 100 000 elements may differ by one rounding
+    step of the storage type at the magnitude of the values that were summed (2^-8 of the largest
+    |value| for bf16, 2^-11 for fp16): y = T(y0 + T(scale * sum)) rounds twice at the magnitude of
+    y0, the kernel and the oracle add up the fp32 sum in different orders, and where y0 and the
+    delta cancel, one flipped rounding is larger than any tolerance relative to the small result."""
+    bad = np.abs(got - want) > atol + rtol * np.abs(want)
+    if not bad.any():
+        return
+    step = float(np.abs(want).max()) * (2.0 ** -8 if dtype == "bf16" else 2.0 ** -11)
+    assert bad.sum() <= max(1, int(2e-5 * bad.size)), f"{bad.sum()} of {bad.size} elements outside rtol/atol"
+    assert np.abs(got - want)[bad].max() <= step, (np.abs(got - want)[bad].max(), step)
+
+
 def oracle_chain(c, p, R, y0=None):
     delta = O.ref_bgmv_shrink(np.zeros((c.batch, R), np.float32), c.x, c.key, c.a_start, c.a_len, c.a_loc, c.bins, p,
                               dtype=c.dtype)
@@ -79,6 +93,12 @@ def oracle_chain(c, p, R, y0=None):
     (4096, [64, 32, 16, 8, 64, 8], 64),
     (5120, [64, 32, 16], 19),
     (768, [128, 8], 9),
+    (4608, [16, 32], 40),          # page widths of the shrink's wider straight-line paths, whole and
+    (6144, [32, 16], 23),          # partial last vector columns, runs of up to four tokens
+    (5632, [16, 32], 30),
+    (8192, [16, 32], 21),
+    (7168, [16], 11),
+    (8704, [32, 16], 9),           # wider than any of them: the general path
 ])
 def test_decode_chain_matches_oracle(gpu, dtype, hidden, ranks, batch):
     c = make_case(100 + hidden + batch, hidden, ranks, batch, dtype=dtype, zipf_alpha=1.0)
@@ -91,8 +111,8 @@ def test_decode_chain_matches_oracle(gpu, dtype, hidden, ranks, batch):
         np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
         # expand is checked on the GPU's own shrink output so one rounding flip in delta is not amplified
         y_ref2 = O.ref_bgmv_expand(y0, d_gpu, c.value, c.a_start, c.a_len, c.a_loc, c.bins, p, c.scales, dtype=dtype)
-        np.testing.assert_allclose(y_gpu, y_ref2, rtol=RTOL, atol=ATOL)
-        np.testing.assert_allclose(y_gpu, y_ref, rtol=2 * RTOL, atol=4 * ATOL)
+        assert_close_but_for_rounding_flips(y_gpu, y_ref2, RTOL, ATOL, dtype)
+        assert_close_but_for_rounding_flips(y_gpu, y_ref, 2 * RTOL, 4 * ATOL, dtype)
 
 
 def test_reference_kernel_test_shapes(gpu):
