@@ -31,10 +31,11 @@ HBM_PEAK_GBS = 8000.0
 # a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
 # None where not measured.
 TRAFFIC_BYTES = {
-    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81403867,  # 75112411 read + 6291456 written
-    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true>"): 71000741,     # the q/k/v launch
-    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281674768,  # 155648888 read + 126025879 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16, 1>"): 142878462,  # 140909310 read + 1969152 written
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81480679,  # 75189223 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70960713,  # the q/k/v launch
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281672559,  # 155646789 read + 126025770 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 1>"): 142091895,  # 140122743 read + 1969152 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 3>"): 174437432,  # 168529976 read + 5907456 written
 }
 
 
@@ -137,7 +138,8 @@ def make_step(w, bufs, mode):
                     fn(l, p)
         return sweep
 
-    sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
+    nv = next((n for n in (8, 10, 12, 16) if w.hidden <= 512 * n), 8)  # the instantiation the library picks
+    sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}, {nv}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
     if fused:
         families = {
             "qkv_shrink": (over_layers(qkv_shrink), sk, L, w.qkv_shrink_bytes()),
@@ -441,7 +443,8 @@ def measure_prefill(args, torch, device):
                           "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                           "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                           "TFLOPs": round(flops / us / 1e6, 1),
-                          "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
+                          "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4),
+                          "traffic": TRAFFIC_BYTES.get(("c3", kname))}
     dom = max((k for n, k in kernels.items() if n != "qkv_shrink"), key=lambda k: k["us_per_launch"])
     out = {
         "metric": "LoRA prefill tokens/s + achieved HBM GB/s (% peak), C3 segmented shrink/expand",
