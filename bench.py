@@ -367,19 +367,22 @@ def free_workload(w, bufs, torch):
     torch.cuda.empty_cache()
 
 
-def measure_prefill(args, torch, device):
-    """C3: q/k/v/o segmented shrink and expand over a prefill batch, per layer.  Returns the
-    JSON object of the prefill workload."""
+def measure_prefill(args, torch, device, w=None, seg=None):
+    """q/k/v/o segmented shrink and expand over a prefill batch, per layer (C3 unless a pool
+    workload and its requests are passed).  Returns the JSON object of the prefill workload."""
     import slora_hip
     import workloads
     L = min(args.layers, 4)
-    w, seg = workloads.c3_prefill(device, n_layers=L)
+    if w is None:
+        w, seg = workloads.c3_prefill(device, n_layers=L)
     T, H, R = seg.n_tokens, w.hidden, w.max_rank
     g = torch.Generator(device=device)
     g.manual_seed(7)
     x = [torch.randn((T, H), generator=g, device=device, dtype=torch.float32).to(w.dtype) for _ in range(L)]
     y = [torch.zeros((T, H), device=device, dtype=w.dtype) for _ in range(L)]
     d = torch.zeros((T, R), device=device, dtype=w.dtype)
+    ty = "F16" if w.dtype == torch.float16 else "BF16"
+    ks = 1 if R <= 32 else (2 if R <= 64 else 4)
     d3 = [torch.zeros((T, R), device=device, dtype=w.dtype) for _ in range(3)]
     t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
 
@@ -434,10 +437,10 @@ def measure_prefill(args, torch, device):
     kernels = {}
     flops1 = seg.flops(w, H)
     for label, sweep, kname, nbytes, flops in (
-            ("shrink", shrink_sweep, "sgmm_shrink_planned_kernel<BF16, 1>", seg.shrink_bytes(w), flops1),
-            ("qkv_shrink", qkv_shrink_sweep, "sgmm_shrink_planned_kernel<BF16, 3>",
+            ("shrink", shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 1>", seg.shrink_bytes(w), flops1),
+            ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3>",
              3 * seg.shrink_bytes(w) - 2 * T * H * 2, 3 * flops1),
-            ("expand", expand_sweep, "sgmm_expand_walk_kernel<BF16, 2>", seg.expand_bytes(w, H), flops1)):
+            ("expand", expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}>", seg.expand_bytes(w, H), flops1)):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
         kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
                           "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
@@ -451,7 +454,8 @@ def measure_prefill(args, torch, device):
         "value": round(T / (ms_step * 1e-3 / L), 1),
         "unit": "tokens/s per layer",
         "n_gpus": 1, "steps": reps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16" if w.dtype == torch.float16 else "bf16", "data": "synthetic",
         "config": {"workload": w.name, "layers": L, "tokens": T, "requests": int(seg.lens_np.size),
                    "launch": args.launch, "launches_per_step": 8 * L + 1},
         "ms_per_step_qkv_fused": round(ms_step_fused, 4),
@@ -719,6 +723,15 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, bufs, torch, args.cpu_reps)
+    if args.workload == "s4" and not args.no_extras:
+        # the prefill half of the mixed S4 step, over the same pool: 4 requests of 256 tokens
+        pf = measure_prefill(argparse.Namespace(layers=min(w.n_layers, 4), steps=10, warmup=3, launch="graph"), torch,
+                             device, w=w, seg=workloads.c4_prefill_segments(w, device))
+        n = pf["config"]["layers"]
+        out["prefill_part"] = {"what": "4 prefill requests of 256 tokens in the same step, same pool",
+                               "ms_per_layer": round(pf["ms_per_step"] / n, 4),
+                               "ms_per_layer_qkv_fused": round(pf["ms_per_step_qkv_fused"] / n, 4),
+                               "decode_ms_per_layer": round(ms_per_step / w.n_layers, 4), "kernels": pf["kernels"]}
     if args.workload == "s2" and not args.no_extras:
         other_modes.update(measure_dropin_direct(w, bufs, torch, args))
         free_workload(w, bufs, torch)

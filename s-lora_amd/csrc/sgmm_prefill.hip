@@ -202,6 +202,68 @@ __device__ __forceinline__ void shrink_k_loop(const uint16_t* const (&xline)[kSh
   if (i + 1 < n) mul_block(c1);
 }
 
+// The same loop with a ring of D blocks, D - 1 of them in flight while one is multiplied
+// (same blocks in the same order: identical sums).  For launches with few workgroups, where
+// a wavefront waits for its own loads and nobody else's fill the compute unit: 1024 tokens
+// of rank 64 take 16 -> 14.5 us, 4096 tokens 25 -> 23.5 us with D = 4.  With every compute
+// unit streaming (C3) the deeper ring is slower (37 -> 44 us): a wavefront's loads return in
+// order, so the weight rows (cache hits) queue behind the activations of the blocks ahead.
+// A load past the last block re-reads it; only multiplications are skipped.
+template <typename T, int NT, int MF, int D>
+__device__ __forceinline__ void shrink_k_loop_ring(const uint16_t* const (&xline)[kShrMF][2],
+                                                   const uint16_t* const (&wline)[4][2], int wave, int piece,
+                                                   int h_in, f32x4 (&acc)[kShrMF][4]) {
+  const int blocks = (h_in + 63) >> 6;
+  const int n = (blocks - wave + kShrWaves - 1) / kShrWaves;  // blocks of this wavefront
+  if (n <= 0) return;
+  const bool ragged_k = (h_in & 63) != 0;
+  struct Block {
+    u32x4 a[MF][2], b[NT][2];
+  };
+  auto load_block = [&](int i, Block& blk) {
+    if (i >= n) i = n - 1;
+    int k = (i * kShrWaves + wave) * 64 + piece * 8;
+    const bool k_in = k < h_in;
+    if (!k_in) k = 0;
+#pragma unroll
+    for (int f = 0; f < MF; ++f)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) blk.a[f][g] = ldg16_stream(xline[f][g] + k);
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) blk.b[t][g] = ldg16(wline[t][g] + k);
+    if (ragged_k && !k_in) {
+#pragma unroll
+      for (int f = 0; f < MF; ++f) blk.a[f][0] = blk.a[f][1] = zero16();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) blk.b[t][0] = blk.b[t][1] = zero16();
+    }
+  };
+  auto mul_block = [&](Block& blk) {
+#pragma unroll
+    for (int f = 0; f < MF; ++f) swap_halves(blk.a[f][0], blk.a[f][1]);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) swap_halves(blk.b[t][0], blk.b[t][1]);
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int f = 0; f < MF; ++f) acc[f][t] = mfma16<T>(blk.a[f][s], blk.b[t][s], acc[f][t]);
+  };
+  Block ring[D];
+#pragma unroll
+  for (int d = 0; d < D - 1; ++d) load_block(d, ring[d]);
+  for (int i = 0; i < n; i += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      load_block(i + d + D - 1, ring[(d + D - 1) % D]);
+      if (i + d < n) mul_block(ring[d]);
+    }
+  }
+}
+
 // The same share of the K loop for q, k and v at once: a 64-k block of the activations is
 // loaded once and multiplied with the block of each projection's weight rows in turn.  Two
 // activation blocks and two weight blocks are held; while one product runs, the weight block
@@ -317,7 +379,7 @@ __device__ __forceinline__ void shrink_k_loop_qkv(const uint16_t* const (&xline)
 // whose weight rows start at a_loc[base_li]; of every 64 rank columns the 16-column
 // tiles t with t % p.col_split == cg.  All threads of the workgroup call it together;
 // it ends with a barrier.
-template <typename T, int NPROJ>
+template <typename T, int NPROJ, bool DEEP>
 __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_part, int64_t row_first, int m_cnt,
                                             int r_eff, int64_t base_li, int rank, int cg) {
   const int cs = p.col_split;
@@ -382,11 +444,20 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
       auto k_loop = [&](auto mf) {
         constexpr int MF = decltype(mf)::value;
         if constexpr (NPROJ == 1) {
-          switch (n_own) {
-            case 1: shrink_k_loop<T, 1, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
-            case 2: shrink_k_loop<T, 2, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
-            case 3: shrink_k_loop<T, 3, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
-            default: shrink_k_loop<T, 4, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+          if (DEEP) {
+            switch (n_own) {
+              case 1: shrink_k_loop_ring<T, 1, MF, 4>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              case 2: shrink_k_loop_ring<T, 2, MF, 4>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              case 3: shrink_k_loop_ring<T, 3, MF, 4>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              default: shrink_k_loop_ring<T, 4, MF, 4>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+            }
+          } else {
+            switch (n_own) {
+              case 1: shrink_k_loop<T, 1, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              case 2: shrink_k_loop<T, 2, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              case 3: shrink_k_loop<T, 3, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+              default: shrink_k_loop<T, 4, MF>(xline, wline[0], wave, piece, p.h_in, acc[0]); break;
+            }
           }
         } else {
           switch (n_own) {
@@ -441,6 +512,7 @@ __device__ __forceinline__ void shrink_tile(const SegShrinkArgs& p, float* s_par
 // 16 token rows: the unit work is shared out in
 constexpr int kShrUnit = 16;
 constexpr int kShrMaxGrid = 256;  // one workgroup per compute unit
+constexpr int kShrDeepTokens = 4096;  // batches up to this size use the deeper K loop (see shrink_k_loop_ring)
 constexpr int kShrChunk = 256;    // requests described at a time (one per thread)
 
 // inclusive prefix sum of `v` over the workgroup; *total receives the sum
@@ -504,7 +576,7 @@ __device__ __forceinline__ int shrink_chunks_needed(int units, int r_eff, uint32
 // read the same weight rows, share an L2) and every workgroup the same cost,
 // whatever the mix of request lengths and ranks.  A workgroup owns the units
 // whose start falls into its part and walks them as tiles of up to kShrMF units.
-template <typename T, int NPROJ>
+template <typename T, int NPROJ, bool DEEP>
 __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   __shared__ int64_t s_wave[kShrWaves];
@@ -698,7 +770,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
               shrink_generic<T>(p, pj, r_eff, base_li + (int64_t)pj * rj, rw0, m0, m_end - m0);
           __syncthreads();
         } else {
-          shrink_tile<T, NPROJ>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, rj, cg);
+          shrink_tile<T, NPROJ, DEEP>(p, s_part, (int64_t)rw0 + m0, m_end - m0, r_eff, base_li, rj, cg);
         }
       }
     }
@@ -792,7 +864,7 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_plan_kernel(int* plan, SegTa
   }
 }
 
-template <typename T, int NPROJ>
+template <typename T, int NPROJ, bool DEEP>
 __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(const SegShrinkArgs p, const int* plan) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   const int slot = (int)(blockIdx.x & 7) * ((int)gridDim.x >> 3) + (int)(blockIdx.x >> 3);
@@ -815,7 +887,7 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(con
           shrink_generic<T>(p, pj, r_eff, base_li + (int64_t)pj * r, row_first, m0, m_cnt);
       __syncthreads();
     } else {
-      shrink_tile<T, NPROJ>(p, s_part, (int64_t)row_first + m0, m_cnt, r_eff, base_li, r, cg);
+      shrink_tile<T, NPROJ, DEEP>(p, s_part, (int64_t)row_first + m0, m_cnt, r_eff, base_li, r, cg);
     }
   }
 }
@@ -1295,7 +1367,9 @@ bool shrink_plan_usable(int64_t n_requests, int64_t m_tiles, int64_t grid, int c
   return grid > 0 && n_requests <= kShrChunk && n_requests <= grid / cs && m_tiles <= 1024;
 }
 
-template <typename T, int NPROJ>
+// DEEP: the instantiation whose single-projection K loop keeps three blocks in flight (for
+// launches with few workgroups, see shrink_k_loop_ring)
+template <typename T, int NPROJ, bool DEEP>
 int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t stream) {
   const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
   int64_t grid = 0;
@@ -1303,8 +1377,8 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
   shrink_geometry(p.t.n_tokens, p.t.n_requests, p.m_tiles, p.max_rank, grid, q.col_split);
   if (grid <= 0) return SLORA_OK;
   if (plan != nullptr && !shrink_plan_usable(p.t.n_requests, p.m_tiles, grid, q.col_split)) return SLORA_ERR_BAD_SHAPE;
-  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ>)
-                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ>);
+  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ, DEEP>)
+                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ, DEEP>);
   static bool attr_done[2] = {false, false};  // benign if two threads race: the call is idempotent
   if (!attr_done[plan != nullptr]) {
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
@@ -1314,10 +1388,10 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
     attr_done[plan != nullptr] = true;
   }
   if (plan != nullptr)
-    hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q,
+    hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ, DEEP>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q,
                        plan);
   else
-    hipLaunchKernelGGL((sgmm_shrink_kernel<T, NPROJ>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
+    hipLaunchKernelGGL((sgmm_shrink_kernel<T, NPROJ, DEEP>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
@@ -1392,8 +1466,13 @@ int seg_shrink_common(const int* plan, bool planned, void* const o[3], int nproj
   p.vec_ok = (h_in % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(x) && aligned16(w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (nproj == 3)
-    return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 3>(p, plan, s) : launch_seg_shrink<BF16, 3>(p, plan, s);
-  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 1>(p, plan, s) : launch_seg_shrink<BF16, 1>(p, plan, s);
+    return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 3, false>(p, plan, s)
+                                    : launch_seg_shrink<BF16, 3, false>(p, plan, s);
+  if (n_tokens <= kShrDeepTokens)
+    return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 1, true>(p, plan, s)
+                                    : launch_seg_shrink<BF16, 1, true>(p, plan, s);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 1, false>(p, plan, s)
+                                  : launch_seg_shrink<BF16, 1, false>(p, plan, s);
 }
 
 }  // namespace

@@ -238,6 +238,26 @@ class PrefillSegments:
         return int(2 * h * (w.ranks[self.ids_np] * self.lens_np).sum())
 
 
+def segments(device, lens, ids) -> PrefillSegments:
+    """Requests of the given lengths and adapters laid end to end."""
+    lens = np.asarray(lens, dtype=np.int32)
+    ids = np.asarray(ids, dtype=np.int64)
+    start = np.zeros(lens.size, np.int32)
+    start[1:] = np.cumsum(lens)[:-1]
+    seg = PrefillSegments(lens_np=lens, ids_np=ids)
+    seg.b_start_loc = torch.from_numpy(start).to(device)
+    seg.b_seq_len = torch.from_numpy(lens).to(device)
+    seg.b_indicies = torch.from_numpy(ids).to(device)
+    return seg
+
+
+def c4_prefill_segments(w, device, seed=4) -> PrefillSegments:
+    """The prefill half of the mixed S4 step: 4 requests of 256 tokens whose adapters are drawn
+    like the decode tokens' (Zipf(0.9) over the workload's adapters)."""
+    rng = np.random.default_rng(seed + 100)
+    return segments(device, [256] * 4, np.sort(zipf_ids(rng, len(w.ranks), 4, 0.9)))
+
+
 def c3_prefill(device, n_layers=4, n_pages=65536, seed=3):
     """64 requests of 8..512 tokens sorted by adapter, 100 adapters of ranks
     {64,32,16,8}, bfloat16, hidden 4096, pages scattered over the pool."""
