@@ -1,7 +1,7 @@
 """Decode shrink / expand on the GPU against the CPU oracle.
 
-Everything goes through the C ABI of libslora_hip.so (the Python mirror of
-``dispatch_bgmv`` is a ctypes call).  Tolerance for floating point is the one
+Everything goes through the C ABI of libslora_hip.so (``slora_hip.dispatch_bgmv`` is the
+compiled extension's check-and-call in front of it).  Tolerance for floating point is the one
 the task states: rtol 1e-2, atol 1e-3 in fp16 and bf16.  Gather/index work is
 checked bit-exactly with integer-valued cases.
 """
