@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define SLORA_VERSION 110 /* 0.1.10: + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed, slora_pool_alloc_contiguous_static */
+#define SLORA_VERSION 101 /* 0.1.1: + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed, slora_pool_alloc_contiguous_static */
 
 #define SLORA_API __attribute__((visibility("default")))
 
