@@ -358,6 +358,29 @@ def measure_dropin_direct(w, bufs, torch, args):
         "host_us_per_call": round(host_us, 2)}}
 
 
+def measure_other_shapes(w, bufs, torch):
+    """The decode step at the S4 and S6 shapes (a few layers each), each in a child process of
+    its own once this process has given its pools back: what the same kernels reach when a
+    launch moves hundreds of megabytes instead of tens."""
+    import subprocess
+    free_workload(w, bufs, torch)
+    res = {}
+    for wl, layers in (("s4", 8), ("s6", 4)):
+        cmd = [sys.executable, os.path.abspath(__file__), "--workload", wl, "--layers", str(layers), "--steps", "10",
+               "--warmup", "3", "--no-cpu-baseline", "--no-extras"]
+        try:
+            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=240)
+            d = json.loads([l for l in proc.stdout.splitlines() if l.startswith("{")][-1])
+            res[wl] = {"workload": d["config"]["workload"], "layers": d["config"]["layers"],
+                       "ms_per_step": d["ms_per_step"], "tokens_per_s": d["value"], "step_hbm": d["step_hbm"],
+                       "kernels": {k: {"us_per_launch": v["us_per_launch"], "frac": v["frac"],
+                                       "kernel_over_ceiling": v.get("read_only_ceiling", {}).get("kernel_over_ceiling")}
+                                   for k, v in d["kernels"].items()}}
+        except Exception as e:  # the headline line is printed whatever happens here
+            res[wl] = {"error": f"{type(e).__name__}: {e}"}
+    return res
+
+
 def free_workload(w, bufs, torch):
     """Give the decode pools back before another workload is built."""
     w.key_buffer.clear()
@@ -741,6 +764,8 @@ def main():
                              "tokens": c3["config"]["tokens"], "dtype": "bf16", "kernels": c3["kernels"]}
     if other_modes:
         out["modes"] = other_modes
+    if args.workload == "s2" and not args.no_extras:
+        out["other_shapes"] = measure_other_shapes(w, bufs, torch)
     print(json.dumps(out), flush=True)
 
 
