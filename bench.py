@@ -61,6 +61,9 @@ def parse_args():
     ap.add_argument("--placement", choices=["scattered", "runs"], default="scattered",
                     help="where the adapters' pages lie in the pool -- scattered (the metric's configuration) "
                          "or one contiguous run per adapter (what MemoryAllocator.alloc_adapter asks for)")
+    ap.add_argument("--keep-plan", action="store_true",
+                    help="planned modes: build the plan once with its item count read back and do not rebuild it "
+                         "inside the step (launches sized exactly; only right while the batch stays the same)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="leave out the 'modes' (reference call pattern, direct launches) and 'prefill_c3' blocks "
@@ -90,7 +93,7 @@ class StepBuffers:
         self.delta = [torch.zeros((B, w.max_rank), device=device, dtype=w.dtype) for _ in range(3)]
 
 
-def make_step(w, bufs, mode):
+def make_step(w, bufs, mode, keep_plan=False):
     """Returns (step, families).  `families` maps a label to (sweep, kernel
     name, launches per sweep, algorithmic bytes per launch): one sweep per kind
     of launch the step issues, over all layers, so that each kind's launch
@@ -154,7 +157,7 @@ def make_step(w, bufs, mode):
         }
 
     def step():
-        if planned:
+        if planned and not keep_plan:
             slora_hip.rebuild_plan(plan, *t, w.n_pages)
         else:
             # a new batch every step: calls that pass no plan may reuse one only within the step
@@ -623,7 +626,7 @@ def main():
         w = workloads.s6_decode(device, n_layers=min(args.layers, 8), batch=args.batch if args.batch != 256 else 1024,
                                 placement=args.placement)
     bufs = StepBuffers(w, device)
-    step, families = make_step(w, bufs, args.mode)
+    step, families = make_step(w, bufs, args.mode, args.keep_plan)
     fused = args.mode.endswith("fused")
     if args.check:
         check_layer0(w, bufs, torch)

@@ -73,6 +73,7 @@ struct Item {
   int j0;        // first row / page of the item inside each projection block
   int more;      // rows beyond the listed ones exist (rank > rank_cap)
   int tok[kTT];  // token indices
+  int plan_items;  // items of the plan the record was read from (0: no plan, or not a plan)
 };
 
 __device__ __forceinline__ int item_token(const Item& it, int t) {
@@ -92,6 +93,7 @@ __device__ __forceinline__ void discover_run(const Tables& t, int batch, int b, 
   it.n_tok = 0;
   it.r = 0;
   it.more = 0;
+  it.plan_items = 0;
   constexpr int kGroup = 8;  // chunks of 64 ids loaded together
   const int64_t a = t.bins[b];
   int64_t v[kGroup];
@@ -182,6 +184,7 @@ __device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx,
   it.tok[2] = t2;
   it.tok[3] = t3;
   const bool ok = (magic == kPlanMagic) & (idx < n_items);
+  it.plan_items = magic == kPlanMagic ? n_items : 0;
   it.a = a;
   it.r = r;
   it.n_tok = ok ? n_tok : 0;
@@ -212,6 +215,7 @@ struct ShrinkArgs {
   Tables t;
   int64_t page_elems;
   int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
+  int strided;  // planned launch with fewer workgroups than the plan may have items (see planned_grid)
 };
 
 // The common case in straight-line code: the whole page in one pass (hidden <= 512 * NV
@@ -304,7 +308,7 @@ __device__ __forceinline__ void shrink_fast(const ShrinkArgs& p, const Item& it,
 // Grid: x = item (planned) or token * blocks + block (stateless), y = projection of the
 // launch.  s_x: [lds_tt][h_in / 8] LDS words.
 template <typename T, bool PLANNED, int NV>
-__device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int proj, u32x4* s_x) {
+__device__ __forceinline__ int shrink_body(const ShrinkArgs& p, int unit, int proj, u32x4* s_x) {
   constexpr int NW = 4;
   constexpr int NTASK = 2;
   constexpr int NT = NW * kWave;
@@ -333,9 +337,9 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
       page2[i] = lookup_page_nobranch(p.t, it.base + (int64_t)it.r * (p.qkvo0 + proj) + it.j0 + jr,
                                       it.n_tok > 0 && p.t.n_loc > 0);
   }
-  if (it.n_tok <= 0) return;
+  if (it.n_tok <= 0) return it.plan_items;
   const int r_eff = it.r < p.y_cols ? it.r : p.y_cols;
-  if (it.j0 >= r_eff) return;  // uniform over the workgroup
+  if (it.j0 >= r_eff) return it.plan_items;  // uniform over the workgroup
 
   const int nvec = p.h_in >> 3;
   if (nvec <= NV * kWave && it.n_tok <= p.lds_tt && !(PLANNED && it.more)) {
@@ -343,7 +347,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
     for (int i = 0; i < 2; ++i)
       if (it.j0 + wave + 4 * i >= r_eff) page2[i] = -1;
     shrink_fast<T, NV>(p, it, proj, r_eff, page2, s_x);
-    return;
+    return it.plan_items;
   }
   const uint16_t* wbase = reinterpret_cast<const uint16_t*>(p.w);
   int row[NTASK];
@@ -455,6 +459,7 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
       }
     }
   }
+  return it.plan_items;
 }
 
 // NV: the straight-line path of this instantiation holds pages of up to 512 * NV elements
@@ -462,7 +467,16 @@ __device__ __forceinline__ void shrink_body(const ShrinkArgs& p, int unit, int p
 template <typename T, bool PLANNED, int NV>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];  // [lds_tt][h_in / 8]
-  shrink_body<T, PLANNED, NV>(p, (int)blockIdx.x, (int)blockIdx.y, s_x);
+  int unit = (int)blockIdx.x;
+  const int n_items = shrink_body<T, PLANNED, NV>(p, unit, (int)blockIdx.y, s_x);
+  if (PLANNED && p.strided) {
+    // a launch sized for a fraction of the plan's capacity: the items beyond the grid, if the
+    // batch has that many, are walked here (uniform over the workgroup)
+    for (unit += (int)gridDim.x; unit < n_items; unit += (int)gridDim.x) {
+      __syncthreads();  // the staging area of the item before is free
+      shrink_body<T, PLANNED, NV>(p, unit, (int)blockIdx.y, s_x);
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -479,6 +493,7 @@ struct ExpandArgs {
   int scales_dtype;
   int batch, x_cols, qkvo0, blocks, y_aligned;
   int interleave;  // one-dimensional grid: the workgroups of an item follow each other (see bgmv_expand_kernel)
+  int strided;     // planned launch with fewer workgroups than the plan may have items (see planned_grid)
   int n_units;     // items (planned) or token blocks (stateless) of the launch
   int h_out[3];
   // pages per rank row of each projection: a rank-r adapter's B^T fills ceil(r * h_out /
@@ -705,7 +720,7 @@ __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const 
 // half: workgroup ids run item-fastest, so with a multiple of 8 items every workgroup of
 // an item lands on XCD item % 8.
 template <typename T, int NPROJ, bool PLANNED>
-__device__ __forceinline__ void expand_body(const ExpandArgs& p, int unit, int sub, uint16_t* s_strip) {
+__device__ __forceinline__ int expand_body(const ExpandArgs& p, int unit, int sub, uint16_t* s_strip) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int proj = sub >> 1;
   const int jr = (sub & 1) * 4 + wave;  // page inside the item's block
@@ -719,10 +734,10 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int unit, int s
     discover_run(p.t, p.batch, b, it);
     it.j0 = (unit - b * p.blocks) * kRB;
   }
-  if (it.n_tok <= 0) return;
+  if (it.n_tok <= 0) return it.plan_items;
   const int r = it.r;
   const int r_eff = r < p.x_cols ? r : p.x_cols;
-  if (r_eff <= 0) return;
+  if (r_eff <= 0) return it.plan_items;
   const int k = it.j0 + jr;
   // pages that hold this projection's h_out * r elements
   const int sh = p.pages_shift[proj];
@@ -743,7 +758,7 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int unit, int s
   else
     extra = it.j0 + kRB >= p.blocks * kRB;
   const bool has_work = k < n_pg || extra;
-  if (!has_work) return;
+  if (!has_work) return it.plan_items;
   const bool pow2 = (r & (r - 1)) == 0;
   // the vector path reads and writes y 16 bytes at a time: rows and page boundaries must fall on multiples of 8 outputs
   const bool vec_ok = pow2 && r >= 8 && r <= 128 && (r_eff & 7) == 0 && (p.x_cols & 7) == 0 &&
@@ -756,6 +771,7 @@ __device__ __forceinline__ void expand_body(const ExpandArgs& p, int unit, int s
 #pragma unroll 1
     for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
   }
+  return it.plan_items;
 }
 
 // ---------------------------------------------------------------------------
@@ -1207,7 +1223,12 @@ __global__ __launch_bounds__(256, NPROJ == 3 ? 5 : 4) void bgmv_expand_kernel(co
     sub = g % S;
     if (unit >= p.n_units) return;
   }
-  expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
+  const int n_items = expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
+  if (PLANNED && p.strided) {  // the items beyond the grid, if the batch has that many
+    const int stride = p.interleave ? (int)gridDim.x / (2 * NPROJ) : (int)gridDim.x;  // units of the grid
+    for (unit += stride; unit < n_items; unit += stride)
+      expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
+  }
 }
 
 template <typename T, int NPROJ, bool PLANNED>
@@ -1236,10 +1257,20 @@ int dispatch_expand(const ExpandArgs& p, int nproj, bool planned, int64_t grid, 
   return planned ? launch_expand<T, 1, true>(p, grid, s) : launch_expand<T, 1, false>(p, grid, s);
 }
 
-// grid of a planned launch: the items the caller read back, else the plan's capacity
-int64_t planned_grid(int64_t n_items, int64_t batch, int64_t rank_cap) {
+// Grid of a planned launch: the items the caller read back.  Without that count (a plan rebuilt
+// in place, or built inside a graph capture) the plan's capacity is the only bound the host
+// has, several times what a batch usually needs, and every workgroup of an item that does not
+// exist still costs its hand-out and one round trip.  Such launches get a quarter of the
+// capacity (a multiple of 8, so that item i stays on XCD i % 8) and their workgroups walk the
+// items in strides of the grid: a usual batch fits the grid, a batch of many short runs makes
+// a workgroup do up to four items one after the other.
+int64_t planned_grid(int64_t n_items, int64_t batch, int64_t rank_cap, int& strided) {
   const int64_t cap = plan_max_items(batch, rank_cap);
-  return (n_items > 0 && n_items < cap) ? n_items : cap;
+  strided = 0;
+  if (n_items > 0 && n_items < cap) return n_items;
+  if (cap <= 64 * kXcds) return cap;
+  strided = 1;
+  return (cap / 4 + kXcds - 1) / kXcds * kXcds;
 }
 
 constexpr int kNothingToDo = 1;  // a valid call with no work; callers turn it into SLORA_OK
@@ -1274,7 +1305,8 @@ int shrink_prepare(const void* plan, int64_t n_items, int64_t rank_cap, void* co
   p.y_cols = (int)y_cols;
   p.qkvo0 = qkvo0;
   p.blocks = (int)((y_cols + kRB - 1) / kRB);
-  grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
+  p.strided = 0;
+  grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap, p.strided) : batch * p.blocks;
   return SLORA_OK;
 }
 
@@ -1349,7 +1381,8 @@ int expand_prepare(const void* plan, int64_t n_items, int64_t rank_cap, void* co
   // stateless: the rank is only known on the device; the grid covers the pages of a rank
   // up to the delta width (an adapter uses min(rank, ceil(h_out*rank/page_elems)) pages)
   p.blocks = (int)((x_cols + kRB - 1) / kRB);
-  grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap) : batch * p.blocks;
+  p.strided = 0;
+  grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap, p.strided) : batch * p.blocks;
   return SLORA_OK;
 }
 

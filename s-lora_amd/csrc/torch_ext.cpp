@@ -49,13 +49,16 @@ int dtype_code(const Tensor& t, const char* what) {
 
 void* stream_of(const Tensor& t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
 
-bool stream_is_capturing(void* stream) {
+// 0 when the stream is not being captured into a graph, else the id of the capture (never 0)
+uint64_t capture_id_of(void* stream) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &st) != hipSuccess) {
+  unsigned long long id = 0;
+  if (hipStreamGetCaptureInfo(static_cast<hipStream_t>(stream), &st, &id) != hipSuccess) {
     (void)hipGetLastError();
-    return false;
+    return 0;
   }
-  return st != hipStreamCaptureStatusNone;
+  if (st == hipStreamCaptureStatusNone) return 0;
+  return id != 0 ? (uint64_t)id : ~(uint64_t)0;
 }
 
 // non-zero return code of the C ABI -> the RuntimeError a TORCH_CHECK of the reference would raise
@@ -191,6 +194,11 @@ void rebuild_plan(const std::shared_ptr<BgmvPlan>& plan, const Tensor& start_ind
               indicies.numel());
   build_plan_into(plan->buf, start_indicies, lora_ranks, loc_indicies, indicies, plan->rank_cap, n_pages,
                   stream_of(indicies), "rebuild_plan");
+  // the new batch's item count is not known on the host (nothing is read back, so that the call can be
+  // recorded into a graph): launches with this plan are sized for its capacity from now on
+  plan->n_items = 0;
+  plan->max_rank = 0;
+  plan->n_runs = 0;
 }
 
 // Plans built on behalf of callers that pass none.  The reference's engine issues all
@@ -215,6 +223,7 @@ class PlanCache {
     hipEvent_t landed = nullptr;
     bool pending = false;
     uint64_t used = 0;
+    uint64_t capture = 0;  // the graph capture the plan was built in (its build is a node of that graph), 0: none
   };
 
   ~PlanCache() {
@@ -227,12 +236,17 @@ class PlanCache {
     streak_ = paused_ = 0;
   }
 
-  // nullptr: no plan for this call (cache off, capturing, inference tensors, cooling down)
+  // nullptr: no plan for this call (cache off, inference tensors, cooling down).
+  // While the stream is being captured into a graph a plan is built and reused as well, within
+  // that capture only: its build kernel becomes a node of the graph, so every replay rebuilds
+  // the plan from what the index tensors hold then, and the buffer comes from the graph's own
+  // memory pool.  Such a plan's item count is never read back (no host copy may be captured
+  // usefully): its launches are sized for the plan's capacity.
   std::shared_ptr<BgmvPlan> get(const Tensor& start_indicies, const Tensor& lora_ranks, const Tensor& loc_indicies,
                                 const Tensor& indicies, int64_t rank_cap, int64_t n_pages, void* stream) {
     if (!g_cache_enabled || indicies.numel() == 0 || rank_cap <= 0 || rank_cap > SLORA_MAX_RANK) return nullptr;
     if (!cacheable({&start_indicies, &lora_ranks, &loc_indicies, &indicies})) return nullptr;
-    if (stream_is_capturing(stream)) return nullptr;
+    const uint64_t capture = capture_id_of(stream);
     std::lock_guard<std::mutex> lock(mu_);
     if (paused_ > 0) {
       --paused_;
@@ -242,11 +256,13 @@ class PlanCache {
     const int device = indicies.get_device();
     ++clock_;
     for (Entry& e : entries_) {
-      if (!e.plan || e.rank_cap != rank_cap || e.n_pages != n_pages || e.stream != stream || e.device != device) continue;
+      if (!e.plan || e.rank_cap != rank_cap || e.n_pages != n_pages || e.stream != stream || e.device != device ||
+          e.capture != capture)
+        continue;
       bool same = true;
       for (int i = 0; i < 4 && same; ++i) same = e.ids[i].matches(*ts[i]);
       if (!same) continue;
-      if (e.pending && hipEventQuery(e.landed) == hipSuccess) {
+      if (e.pending && capture == 0 && hipEventQuery(e.landed) == hipSuccess) {
         e.pending = false;
         e.plan->n_items = e.host_head[1];
         e.plan->max_rank = e.host_head[2];
@@ -264,9 +280,13 @@ class PlanCache {
     }
     // build into the least recently used slot
     if ((int)entries_.size() < kCapacity) entries_.emplace_back();
-    Entry* slot = &entries_[0];
-    for (Entry& e : entries_)
-      if (!e.plan) { slot = &e; break; } else if (e.used < slot->used) slot = &e;
+    Entry* slot = nullptr;
+    for (Entry& e : entries_) {
+      if (capture != 0 && e.pending) continue;  // no waiting for a copy while a graph is being captured
+      if (!e.plan) { slot = &e; break; }
+      if (slot == nullptr || e.used < slot->used) slot = &e;
+    }
+    if (slot == nullptr) return nullptr;
     if (slot->pending) {  // its copy may still be in flight: wait for it before the words are reused
       (void)hipEventSynchronize(slot->landed);
       slot->pending = false;
@@ -277,16 +297,17 @@ class PlanCache {
     plan->buf = alloc_plan_buffer(plan->batch, rank_cap, indicies, "dispatch_bgmv (plan)");
     build_plan_into(plan->buf, start_indicies, lora_ranks, loc_indicies, indicies, rank_cap, n_pages, stream,
                     "dispatch_bgmv (plan)");
-    if (slot->host_head == nullptr) {
+    if (capture == 0 && slot->host_head == nullptr) {
       void* p = nullptr;
       if (hipHostMalloc(&p, 8 * sizeof(int32_t), hipHostMallocDefault) == hipSuccess) slot->host_head = static_cast<int32_t*>(p);
       else (void)hipGetLastError();
     }
-    if (slot->landed == nullptr && hipEventCreateWithFlags(&slot->landed, hipEventDisableTiming) != hipSuccess) {
+    if (capture == 0 && slot->landed == nullptr &&
+        hipEventCreateWithFlags(&slot->landed, hipEventDisableTiming) != hipSuccess) {
       (void)hipGetLastError();
       slot->landed = nullptr;
     }
-    if (slot->host_head != nullptr && slot->landed != nullptr &&
+    if (capture == 0 && slot->host_head != nullptr && slot->landed != nullptr &&
         hipMemcpyAsync(slot->host_head, plan->buf.data_ptr(), 8 * sizeof(int32_t), hipMemcpyDeviceToHost,
                        static_cast<hipStream_t>(stream)) == hipSuccess &&
         hipEventRecord(slot->landed, static_cast<hipStream_t>(stream)) == hipSuccess) {
@@ -299,6 +320,7 @@ class PlanCache {
     slot->n_pages = n_pages;
     slot->stream = stream;
     slot->device = device;
+    slot->capture = capture;
     slot->plan = plan;
     slot->used = clock_;
     ++builds_;
@@ -554,6 +576,7 @@ class PrefillPlanCache {
     int device = -1;
     std::shared_ptr<SgmmPlan> plan;
     uint64_t used = 0;
+    uint64_t capture = 0;  // as in PlanCache::Entry
   };
   void clear() {
     std::lock_guard<std::mutex> lock(mu_);
@@ -567,7 +590,7 @@ class PrefillPlanCache {
         max_input_len <= 0)
       return nullptr;
     if (!cacheable({&b_lora_start, &b_lora_ranks, &b_start_loc, &b_seq_len, &b_indicies})) return nullptr;
-    if (stream_is_capturing(stream)) return nullptr;
+    const uint64_t capture = capture_id_of(stream);  // a plan built inside a capture serves that capture only
     std::lock_guard<std::mutex> lock(mu_);
     if (paused_ > 0) {
       --paused_;
@@ -578,7 +601,7 @@ class PrefillPlanCache {
     ++clock_;
     for (Entry& e : entries_) {
       if (e.n_tokens != n_tokens || e.max_rank != max_rank || e.max_input_len != max_input_len || e.stream != stream ||
-          e.device != device)
+          e.device != device || e.capture != capture)
         continue;
       bool same = true;
       for (int i = 0; i < 5 && same; ++i) same = e.ids[i].matches(*ts[i]);
@@ -605,6 +628,7 @@ class PrefillPlanCache {
     slot->max_input_len = max_input_len;
     slot->stream = stream;
     slot->device = device;
+    slot->capture = capture;
     slot->used = clock_;
     ++builds_;
     return slot->plan;
