@@ -139,8 +139,10 @@ SLORA_API int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_
 
 /* slora_bgmv_shrink / slora_bgmv_shrink_qkv with a plan.  nproj = 1: y0 and
  * qkvo as in slora_bgmv_shrink; nproj = 3: y0,y1,y2 = q,k,v and qkvo = 0.
- * n_items = 0 launches for the plan's capacity (always enough); a caller that
- * read the item count back passes it. */
+ * n_items: the item count a caller read back (one workgroup per item), or 0:
+ * the launch then has a quarter of the plan's capacity in workgroups, which
+ * walk the items in strides of the grid -- right for any batch the plan may
+ * hold, and the form to record into a graph that is replayed over new batches. */
 SLORA_API int slora_bgmv_shrink_planned(const void* plan, int64_t rank_cap, int64_t n_items, int nproj,
                                         void* y0, void* y1, void* y2, const void* x, const void* w,
                                         const slora_tables* tables, const int64_t* bins,
