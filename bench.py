@@ -31,11 +31,11 @@ HBM_PEAK_GBS = 8000.0
 # a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
 # None where not measured.
 TRAFFIC_BYTES = {
-    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81480679,  # 75189223 read + 6291456 written
-    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70960713,  # the q/k/v launch
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81508234,  # 75216778 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70977970,  # the q/k/v launch
     ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281672559,  # 155646789 read + 126025770 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16, 1>"): 142091895,  # 140122743 read + 1969152 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16, 3>"): 174437432,  # 168529976 read + 5907456 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 1, false>"): 142091895,  # 140122743 read + 1969152 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 3, false>"): 174437432,  # 168529976 read + 5907456 written
 }
 
 
@@ -463,8 +463,9 @@ def measure_prefill(args, torch, device, w=None, seg=None):
     kernels = {}
     flops1 = seg.flops(w, H)
     for label, sweep, kname, nbytes, flops in (
-            ("shrink", shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 1>", seg.shrink_bytes(w), flops1),
-            ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3>",
+            ("shrink", shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 1, {'true' if T <= 4096 else 'false'}>",
+             seg.shrink_bytes(w), flops1),
+            ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3, false>",
              3 * seg.shrink_bytes(w) - 2 * T * H * 2, 3 * flops1),
             ("expand", expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}>", seg.expand_bytes(w, H), flops1)):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
