@@ -147,3 +147,41 @@ def test_prefill_step_in_a_graph(gpu, how):
         for p in range(4):
             assert torch.equal(y[p], want[p]), (how, rep, p)
     slora_hip.clear_prefill_plan_cache()
+
+
+@pytest.mark.parametrize("kv_out", [256, 64])
+def test_plan_without_item_count_walks_every_item(gpu, kv_out):
+    """A plan whose item count the host does not have (readback=False, as after rebuild_plan or
+    inside a capture) is launched with a quarter of its capacity in workgroups.  Here nearly
+    every token has an adapter of its own, so the batch has close to the capacity in items and
+    every workgroup walks several of them; with k/v narrower than a page the expand also
+    uses its interleaved grid.  Bitwise the results of the plan-free calls."""
+    import slora_hip
+    from slora_hip import dispatch_bgmv, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_shrink
+    n_ad, batch, H, R = 300, 600, 256, 16
+    rng = np.random.default_rng(3)
+    bins = np.concatenate([np.arange(n_ad), rng.integers(0, n_ad, size=batch - n_ad)])
+    rng.shuffle(bins)
+    c = make_case(77, H, [R] * n_ad, batch, dtype="bf16", bins=bins, h_out=[H, kv_out, kv_out, H])
+    g = GpuCase(c, gpu)
+    t = (g.a_start, g.a_len, g.a_loc, g.bins)
+    plan = slora_hip.make_plan(*t, R, c.n_pages, False)
+    assert plan.n_items == 0
+    d = [torch.zeros((batch, R), dtype=g.tdt, device=gpu) for _ in range(3)]
+    y0 = [torch.randn((batch, h), device=gpu).to(g.tdt) for h in c.h_out]
+    y = [t_.clone() for t_ in y0]
+    dispatch_bgmv_qkv_shrink(d[0], d[1], d[2], g.x, g.key, *t, plan=plan)
+    dispatch_bgmv_qkv_expand(y[0], y[1], y[2], d[0], d[1], d[2], g.value, *t, g.scales, plan=plan)
+    do = torch.zeros((batch, R), dtype=g.tdt, device=gpu)
+    dispatch_bgmv(do, g.x, g.key, *t, 3, g.scales, plan=plan)
+    dispatch_bgmv(y[3], do, g.value, *t, 3, g.scales, plan=plan)
+    torch.cuda.synchronize()
+    head = plan.buf[:8].cpu().tolist()
+    assert head[1] > (batch * 2) // 4          # more items than a quarter of the capacity (2 per token)
+    for p in range(4):
+        dd = torch.zeros((batch, R), dtype=g.tdt, device=gpu)
+        yy = y0[p].clone()
+        dispatch_bgmv(dd, g.x, g.key, *t, p, g.scales, plan=False)
+        dispatch_bgmv(yy, dd, g.value, *t, p, g.scales, plan=False)
+        assert torch.equal(d[p] if p < 3 else do, dd), p
+        assert torch.equal(y[p], yy), p
