@@ -43,7 +43,8 @@ class LoraUnorderedBatchInfer:
     """One object per batch, as in the reference (model_rpc.py:234 builds it per step).
 
     ``infer_adapter``: the tables ``a_loc / a_start / a_len / a_scaling``, ``adapter_dirs`` /
-    ``idx_map`` and ``mem_manager.key_buffer / value_buffer`` (``slora_hip.InferAdapter`` or
+    ``idx_map`` and the pool as ``mem_manager.key_buffer / value_buffer`` or, like the reference's
+    ``NaiveInferAdapter``, as ``key_buffer / value_buffer`` of its own (``slora_hip.InferAdapter`` or
     anything with those attributes).  ``adapters``: per request an object with ``lora_dir``
     and ``r`` (the reference's ``LoraTpPartAdapter``); ``None`` entries (requests on the bare
     base model, which the reference does not support either, :35-36) are rejected."""
@@ -53,9 +54,11 @@ class LoraUnorderedBatchInfer:
         if any(a is None for a in adapters):
             raise ValueError("requests without an adapter are not supported (as in the reference)")
         self.infer_adapter = infer_adapter
-        mm = infer_adapter.mem_manager
-        self.key_buffer: List[torch.Tensor] = mm.key_buffer
-        self.value_buffer: List[torch.Tensor] = mm.value_buffer
+        # the pool's buffers: on the adapter table itself (the reference's NaiveInferAdapter, :28-30)
+        # or on its memory manager (:31-33)
+        owner = infer_adapter if hasattr(infer_adapter, "key_buffer") else infer_adapter.mem_manager
+        self.key_buffer: List[torch.Tensor] = owner.key_buffer
+        self.value_buffer: List[torch.Tensor] = owner.value_buffer
         dev = self.key_buffer[0].device
         self.max_lora_dim = max((int(a.r) for a in adapters), default=0)
         idx_map = getattr(infer_adapter, "idx_map", None)

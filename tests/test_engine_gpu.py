@@ -155,6 +155,27 @@ def test_prefill_step_kernel_choice_and_results(gpu, lens, segmented):
             close(res[True][l][p], m.ref(l, p, base[l][p], xin, bins))
 
 
+def test_engine_takes_buffers_from_the_adapter_table_itself(gpu):
+    """The reference's NaiveInferAdapter keeps key_buffer / value_buffer on itself
+    (lora_unordered_batch_infer.py:28-30); such an object works as well."""
+    from types import SimpleNamespace
+    from slora_hip import LoraUnorderedBatchInfer
+    m = _Model(gpu, "f16", 256, 256, 1, {"a": 8, "b": 16})
+    naive = SimpleNamespace(a_loc=m.ia.a_loc, a_start=m.ia.a_start, a_len=m.ia.a_len, a_scaling=m.ia.a_scaling,
+                            adapter_dirs=m.ia.adapter_dirs, key_buffer=m.mm.key_buffer, value_buffer=m.mm.value_buffer)
+    req = ["b", "a", "a", "b", "b"]
+    bins = np.array([m.names.index(n) for n in req])
+    eng = LoraUnorderedBatchInfer(naive, [m.adapters[n] for n in req])
+    assert eng.req_bins.cpu().tolist() == bins.tolist()      # found by searching adapter_dirs, as the reference does
+    eng.begin_step(torch.zeros(5, dtype=torch.int32, device=gpu), torch.full((5,), 9, dtype=torch.int32, device=gpu),
+                   is_prefill=False, max_b_seq_len=9)
+    rng = np.random.default_rng(2)
+    x, base = _inputs(m, rng, 5)
+    out = _run_layers(m, eng, gpu, x, base)
+    for p in range(4):
+        close(out[0][p], m.ref(0, p, base[0][p], x[0][1] if p == 3 else x[0][0], bins))
+
+
 def test_engine_rejects_requests_without_adapter(gpu):
     from slora_hip import LoraUnorderedBatchInfer
     m = _Model(gpu, "f16", 256, 256, 1, {"a": 8})
