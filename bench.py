@@ -33,7 +33,8 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES = {
     ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81508234,  # 75216778 read + 6291456 written
     ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70977970,  # the q/k/v launch
-    ("c3", "sgmm_expand_walk_kernel<BF16, 2>"): 281672559,  # 155646789 read + 126025770 written
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 1>"): 281697148,  # 155671241 read + 126025907 written
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 3>"): 860966846,  # 482889526 read + 378077320 written
     ("c3", "sgmm_shrink_planned_kernel<BF16, 1, false>"): 142091895,  # 140122743 read + 1969152 written
     ("c3", "sgmm_shrink_planned_kernel<BF16, 3, false>"): 174437432,  # 168529976 read + 5907456 written
 }
@@ -410,6 +411,7 @@ def measure_prefill(args, torch, device, w=None, seg=None):
     ty = "F16" if w.dtype == torch.float16 else "BF16"
     ks = 1 if R <= 32 else (2 if R <= 64 else 4)
     d3 = [torch.zeros((T, R), device=device, dtype=w.dtype) for _ in range(3)]
+    y3 = [[torch.zeros((T, H), device=device, dtype=w.dtype) for _ in range(3)] for _ in range(L)]  # q, k, v outputs
     t = (w.a_loc, w.a_start, w.a_len, seg.b_start_loc, seg.b_seq_len, seg.b_indicies)
 
     def plan():  # once per prefill step, as the automatic cache does for a caller that passes none
@@ -436,13 +438,18 @@ def measure_prefill(args, torch, device, w=None, seg=None):
                 slora_hip.lora_get_qkvo_fwd_expand(d, w.value_buffer[l].view(-1, H), y[l], w.a_scaling, *t, H, p, R,
                                                    seg.max_len)
 
-    def step_fused():  # x read once for q, k and v: 6 launches per layer
+    def qkv_expand_sweep():
+        for l in range(L):
+            for _ in range(4):
+                slora_hip.lora_get_qkvo_fwd_expand_qkv(*d3, w.value_buffer[l].view(-1, H), *y3[l], w.a_scaling, *t, H, H,
+                                                       R, seg.max_len)
+
+    def step_fused():  # q, k and v in one shrink launch (x read once) and one expand launch: 4 launches per layer
         pl = plan()
         for l in range(L):
             key, val = w.key_buffer[l].view(-1, H), w.value_buffer[l].view(-1, H)
             slora_hip.lora_get_qkvo_fwd_shrink_qkv(x[l], key, *d3, *t, H, R, seg.max_len, plan=pl)
-            for p in range(3):
-                slora_hip.lora_get_qkvo_fwd_expand(d3[p], val, y[l], w.a_scaling, *t, H, p, R, seg.max_len)
+            slora_hip.lora_get_qkvo_fwd_expand_qkv(*d3, val, *y3[l], w.a_scaling, *t, H, H, R, seg.max_len)
             slora_hip.lora_get_qkvo_fwd_shrink(x[l], key, d, *t, H, 3, R, seg.max_len, plan=pl)
             slora_hip.lora_get_qkvo_fwd_expand(d, val, y[l], w.a_scaling, *t, H, 3, R, seg.max_len)
 
@@ -467,7 +474,9 @@ def measure_prefill(args, torch, device, w=None, seg=None):
              seg.shrink_bytes(w), flops1),
             ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3, false>",
              3 * seg.shrink_bytes(w) - 2 * T * H * 2, 3 * flops1),
-            ("expand", expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}>", seg.expand_bytes(w, H), flops1)):
+            ("expand", expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}, 1>", seg.expand_bytes(w, H), flops1),
+            ("qkv_expand", qkv_expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}, 3>", 3 * seg.expand_bytes(w, H),
+             3 * flops1)):
         us = time_region(wrap(sweep), reps, 3, torch) * 1e3 / (4 * L)
         kernels[label] = {"kernel": kname, "launches_per_step": 4 * L, "us_per_launch": round(us, 3),
                           "bytes_per_launch": nbytes, "GBps": round(nbytes / us / 1e3, 1),
@@ -475,7 +484,7 @@ def measure_prefill(args, torch, device, w=None, seg=None):
                           "TFLOPs": round(flops / us / 1e6, 1),
                           "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4),
                           "traffic": TRAFFIC_BYTES.get(("c3", kname))}
-    dom = max((k for n, k in kernels.items() if n != "qkv_shrink"), key=lambda k: k["us_per_launch"])
+    dom = max((k for n, k in kernels.items() if not n.startswith("qkv_")), key=lambda k: k["us_per_launch"])
     out = {
         "metric": "LoRA prefill tokens/s + achieved HBM GB/s (% peak), C3 segmented shrink/expand",
         "value": round(T / (ms_step * 1e-3 / L), 1),

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define SLORA_VERSION 101 /* 0.1.1: + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed, slora_pool_alloc_contiguous_static */
+#define SLORA_VERSION 102 /* 0.1.2: + slora_sgmm_expand_qkv; 0.1.1: + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed, slora_pool_alloc_contiguous_static */
 
 #define SLORA_API __attribute__((visibility("default")))
 
@@ -227,6 +227,21 @@ SLORA_API int slora_sgmm_expand(void* o, const void* x, const void* w, const slo
                       int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
                       int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo,
                       int dtype, void* stream);
+
+/* Prefill expand of q, k and v in ONE launch.  The reference issues three expand calls per
+ * layer (slora/models/peft/lora_unordered_batch_infer.py:349-372, 383-398, 409-424); here the
+ * output groups of the three projections share one grid, so a layer pays one launch instead of
+ * three.  x_q / x_k / x_v are three [n_tokens, >= max_rank] inputs with one row stride; o_k and
+ * o_v share width (feat_out_kv, narrower than feat_out_q in grouped-query models) and row
+ * stride.  Per projection the results are those of slora_sgmm_expand with qkvo = 0, 1, 2 and
+ * the same page_elems, bit for bit.  page_elems == 0: feat_out_q. */
+SLORA_API int slora_sgmm_expand_qkv(void* o_q, void* o_k, void* o_v, const void* x_q, const void* x_k, const void* x_v,
+                          const void* w, const slora_tables* tables, const void* scales, int scales_dtype,
+                          const int32_t* b_start_loc, const int32_t* b_seq_len, const int64_t* b_indicies,
+                          int64_t n_requests, int64_t max_input_len, int64_t n_tokens, int64_t feat_out_q,
+                          int64_t feat_out_kv, int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
+                          int64_t w_row_stride, int64_t o_row_stride_q, int64_t o_row_stride_kv, int64_t n_pages,
+                          int dtype, void* stream);
 
 /* ---- moving adapters in and out of the pool --------------------------------- */
 

@@ -907,7 +907,32 @@ struct SegExpandArgs {
   int feat_out, max_rank, qkvo, m_tiles, m_span, n_chunks;
   int vec_ok;
   int row_cap;  // rows of a request at or past this are not touched (max_input_len, rounded up to a row tile)
+  // q, k and v in one launch (nproj == 3): n_chunks counts the output groups of all three, projection
+  // pj owning groups chunk_end[pj - 1] .. chunk_end[pj]; o, x, feat_out, o_stride and qkvo above are then
+  // taken from these by the workgroup (expand_select)
+  int nproj;
+  int chunk_end[3];
+  void* o3[3];
+  const void* x3[3];
+  int feat3[3];
+  int64_t o_stride3[3];
 };
+
+// The arguments as one projection's workgroup sees them, and its output group inside that projection.
+template <int NPROJ>
+__device__ __forceinline__ SegExpandArgs expand_select(const SegExpandArgs& in, int& group) {
+  SegExpandArgs p = in;
+  if (NPROJ == 3) {
+    const int pj = group >= in.chunk_end[1] ? 2 : (group >= in.chunk_end[0] ? 1 : 0);
+    group -= pj == 0 ? 0 : in.chunk_end[pj - 1];
+    p.o = pj == 2 ? in.o3[2] : (pj == 1 ? in.o3[1] : in.o3[0]);
+    p.x = pj == 2 ? in.x3[2] : (pj == 1 ? in.x3[1] : in.x3[0]);
+    p.feat_out = pj == 2 ? in.feat3[2] : (pj == 1 ? in.feat3[1] : in.feat3[0]);
+    p.o_stride = pj == 2 ? in.o_stride3[2] : (pj == 1 ? in.o_stride3[1] : in.o_stride3[0]);
+    p.qkvo = pj;
+  }
+  return p;
+}
 
 constexpr int kExpThreads = 256;
 constexpr int kExpWaves = kExpThreads / kWave;  // 4 wavefronts, one 64-output block each
@@ -1167,15 +1192,16 @@ __device__ __forceinline__ void expand_mfma(const SegExpandArgs& p, int r, int r
 // w takes the group's w-th block of 64 outputs, keeps that block's B^T fragments
 // and walks the span's row tiles, so the four wavefronts together read and write
 // 512 contiguous bytes of every row.
-template <typename T, int KS>
-__global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p) {
+template <typename T, int KS, int NPROJ>
+__global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpandArgs p_all) {
   const int wave = threadIdx.x >> 6;
   // the output group is the fastest index: consecutive workgroup ids go to
   // the 8 XCDs in turn, so every XCD owns 1/8 of the output columns of ALL
   // requests -- disjoint pieces of B^T per L2 and an even share of the y traffic
   int blk = blockIdx.x;
-  const int group = blk % p.n_chunks;
-  blk /= p.n_chunks;
+  int group = blk % p_all.n_chunks;
+  blk /= p_all.n_chunks;
+  const SegExpandArgs p = expand_select<NPROJ>(p_all, group);
   const int req = blk / p.m_tiles;
   const int m0 = (blk - req * p.m_tiles) * p.m_span;
   // The request's three entries are independent loads: all go out before the first
@@ -1217,8 +1243,8 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_kernel(const SegExpan
 // of that line, request by request.
 constexpr int kExpReqs = 256;
 
-template <typename T, int KS>
-__global__ __launch_bounds__(kExpThreads) void sgmm_expand_walk_kernel(const SegExpandArgs p) {
+template <typename T, int KS, int NPROJ>
+__global__ __launch_bounds__(kExpThreads) void sgmm_expand_walk_kernel(const SegExpandArgs p_all) {
   extern __shared__ __align__(16) char s_delta[];
   __shared__ int s_row0[kExpReqs], s_rows[kExpReqs], s_rank[kExpReqs], s_tile0[kExpReqs];
   __shared__ int64_t s_base[kExpReqs];
@@ -1227,8 +1253,9 @@ __global__ __launch_bounds__(kExpThreads) void sgmm_expand_walk_kernel(const Seg
   __shared__ int s_first;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int group = (int)blockIdx.x % p.n_chunks;
-  const int slice = (int)blockIdx.x / p.n_chunks, slices = (int)gridDim.x / p.n_chunks;
+  int group = (int)blockIdx.x % p_all.n_chunks;
+  const int slice = (int)blockIdx.x / p_all.n_chunks, slices = (int)gridDim.x / p_all.n_chunks;
+  const SegExpandArgs p = expand_select<NPROJ>(p_all, group);
 
   // request tid: an invalid one re-reads entry 0 and gets no tiles
   const bool mine = tid < p.t.n_requests;
@@ -1395,10 +1422,10 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
-template <typename T, int KS>
+template <typename T, int KS, int NPROJ>
 int launch_seg_expand_ks(const SegExpandArgs& p, int64_t grid, hipStream_t stream) {
   const bool walk = p.t.n_requests <= kExpReqs && p.t.n_tokens <= (1 << 22);  // tile counts stay far inside 32 bits
-  auto kernel = walk ? sgmm_expand_walk_kernel<T, KS> : sgmm_expand_kernel<T, KS>;
+  auto kernel = walk ? sgmm_expand_walk_kernel<T, KS, NPROJ> : sgmm_expand_kernel<T, KS, NPROJ>;
   constexpr int lds = 2 * kExpChunkRows * kExpLdsRow<KS>;  // 68 KiB for ranks up to 128
   static bool attr_done[2] = {lds <= 64 * 1024, lds <= 64 * 1024};  // benign if two threads race: the call is idempotent
   if (!attr_done[walk]) {
@@ -1425,9 +1452,14 @@ int launch_seg_expand(const SegExpandArgs& p, hipStream_t stream) {
   const int64_t grid = (int64_t)p.t.n_requests * p.m_tiles * p.n_chunks;
   if (grid <= 0) return SLORA_OK;
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
-  if (p.max_rank <= 32) return launch_seg_expand_ks<T, 1>(p, grid, stream);
-  if (p.max_rank <= 64) return launch_seg_expand_ks<T, 2>(p, grid, stream);
-  return launch_seg_expand_ks<T, 4>(p, grid, stream);
+  if (p.nproj == 3) {
+    if (p.max_rank <= 32) return launch_seg_expand_ks<T, 1, 3>(p, grid, stream);
+    if (p.max_rank <= 64) return launch_seg_expand_ks<T, 2, 3>(p, grid, stream);
+    return launch_seg_expand_ks<T, 4, 3>(p, grid, stream);
+  }
+  if (p.max_rank <= 32) return launch_seg_expand_ks<T, 1, 1>(p, grid, stream);
+  if (p.max_rank <= 64) return launch_seg_expand_ks<T, 2, 1>(p, grid, stream);
+  return launch_seg_expand_ks<T, 4, 1>(p, grid, stream);
 }
 
 int seg_shrink_common(const int* plan, bool planned, void* const o[3], int nproj, const void* x, const void* w,
@@ -1473,6 +1505,78 @@ int seg_shrink_common(const int* plan, bool planned, void* const o[3], int nproj
                                     : launch_seg_shrink<BF16, 1, true>(p, plan, s);
   return dtype == SLORA_DTYPE_F16 ? launch_seg_shrink<F16, 1, false>(p, plan, s)
                                   : launch_seg_shrink<BF16, 1, false>(p, plan, s);
+}
+
+// One projection (nproj 1: o[0], x[0], feat_out[0], o_row_stride[0], any qkvo) or q, k and v in one
+// launch (nproj 3, qkvo 0): the output groups of the three projections side by side in one grid.
+int seg_expand_common(void* const o[3], const void* const x[3], int nproj, const void* w, const slora_tables* tables,
+                      const void* scales, int scales_dtype, const int32_t* b_start_loc, const int32_t* b_seq_len,
+                      const int64_t* b_indicies, int64_t n_requests, int64_t max_input_len, int64_t n_tokens,
+                      const int64_t feat_out[3], int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
+                      int64_t w_row_stride, const int64_t o_row_stride[3], int64_t n_pages, int qkvo, int dtype,
+                      void* stream) {
+  if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
+  if (scales_dtype != SLORA_DTYPE_F16 && scales_dtype != SLORA_DTYPE_BF16 && scales_dtype != SLORA_DTYPE_F32)
+    return SLORA_ERR_BAD_DTYPE;
+  if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || max_rank < 0 || page_elems < 0) return SLORA_ERR_BAD_SHAPE;
+  for (int i = 0; i < nproj; ++i)
+    if (feat_out[i] < 0) return SLORA_ERR_BAD_SHAPE;
+  if (qkvo < 0 || qkvo + nproj > 4) return SLORA_ERR_BAD_SHAPE;
+  if (page_elems == 0) page_elems = feat_out[0];  // the reference's convention: page width == output width
+  if (x_row_stride < max_rank || w_row_stride < page_elems) return SLORA_ERR_BAD_SHAPE;
+  int64_t feat_max = 0;
+  for (int i = 0; i < nproj; ++i) {
+    if (o_row_stride[i] < feat_out[i]) return SLORA_ERR_BAD_SHAPE;
+    if (feat_out[i] > feat_max) feat_max = feat_out[i];
+  }
+  if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0 || feat_max == 0) return SLORA_OK;
+  if (max_input_len > n_tokens) max_input_len = n_tokens;  // no request is longer than the batch
+  SegExpandArgs p{};
+  int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
+  if (rc != SLORA_OK) return rc;
+  if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
+  if (w == nullptr || scales == nullptr) return SLORA_ERR_NULL_POINTER;
+  for (int i = 0; i < nproj; ++i)
+    if (feat_out[i] > 0 && (o[i] == nullptr || x[i] == nullptr)) return SLORA_ERR_NULL_POINTER;
+  if (feat_max > (1 << 21) || max_rank > SLORA_MAX_RANK || page_elems > (1LL << 30)) return SLORA_ERR_UNSUPPORTED;
+  p.o = o[0];
+  p.x = x[0];
+  p.w = w;
+  p.scales = scales;
+  p.scales_dtype = scales_dtype;
+  p.x_stride = x_row_stride;
+  p.w_stride = w_row_stride;
+  p.o_stride = o_row_stride[0];
+  p.page_elems = page_elems;
+  p.feat_out = (int)feat_out[0];
+  p.max_rank = (int)max_rank;
+  p.qkvo = qkvo;
+  p.nproj = nproj;
+  p.vec_ok = (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) && aligned16(w);
+  int64_t chunks = 0;
+  for (int i = 0; i < 3; ++i) {
+    if (i < nproj) {
+      chunks += (feat_out[i] + kExpGroup - 1) / kExpGroup;
+      p.o3[i] = o[i];
+      p.x3[i] = x[i];
+      p.feat3[i] = (int)feat_out[i];
+      p.o_stride3[i] = o_row_stride[i];
+      if (feat_out[i] > 0)
+        p.vec_ok = p.vec_ok && (feat_out[i] % 8 == 0) && (o_row_stride[i] % 8 == 0) && aligned16(o[i]) && aligned16(x[i]);
+    }
+    p.chunk_end[i] = (int)chunks;
+  }
+  p.n_chunks = (int)chunks;
+  // rows a workgroup walks: up to kExpSpanTiles tiles, fewer while that leaves the chip short of workgroups
+  int64_t tiles = kExpSpanTiles;
+  while (tiles > 1 &&
+         n_requests * ((max_input_len + kExpTMW * tiles - 1) / (kExpTMW * tiles)) * p.n_chunks < kExpMinGrid)
+    tiles >>= 1;
+  p.m_span = (int)(kExpTMW * tiles);
+  p.row_cap = max_input_len > (1 << 30) ? (1 << 30) : (int)((max_input_len + kExpTMW - 1) / kExpTMW * kExpTMW);
+  p.m_tiles = (int)((max_input_len + p.m_span - 1) / p.m_span);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  return dtype == SLORA_DTYPE_F16 ? launch_seg_expand<F16>(p, s) : launch_seg_expand<BF16>(p, s);
 }
 
 }  // namespace
@@ -1552,48 +1656,28 @@ int slora_sgmm_expand(void* o, const void* x, const void* w, const slora_tables*
                       int64_t feat_out, int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
                       int64_t w_row_stride, int64_t o_row_stride, int64_t n_pages, int qkvo, int dtype,
                       void* stream) {
-  using namespace slora;
-  if (dtype != SLORA_DTYPE_F16 && dtype != SLORA_DTYPE_BF16) return SLORA_ERR_BAD_DTYPE;
-  if (scales_dtype != SLORA_DTYPE_F16 && scales_dtype != SLORA_DTYPE_BF16 && scales_dtype != SLORA_DTYPE_F32)
-    return SLORA_ERR_BAD_DTYPE;
-  if (n_requests < 0 || max_input_len < 0 || n_tokens < 0 || feat_out < 0 || max_rank < 0 || page_elems < 0)
-    return SLORA_ERR_BAD_SHAPE;
-  if (qkvo < 0 || qkvo > 3) return SLORA_ERR_BAD_SHAPE;
-  if (page_elems == 0) page_elems = feat_out;  // the reference's convention: page width == output width
-  if (x_row_stride < max_rank || w_row_stride < page_elems || o_row_stride < feat_out) return SLORA_ERR_BAD_SHAPE;
-  if (n_requests == 0 || max_input_len == 0 || n_tokens == 0 || max_rank == 0 || feat_out == 0) return SLORA_OK;
-  if (max_input_len > n_tokens) max_input_len = n_tokens;  // no request is longer than the batch
-  SegExpandArgs p{};
-  int rc = fill_seg_tables(p.t, tables, b_start_loc, b_seq_len, b_indicies, n_requests, n_tokens, n_pages);
-  if (rc != SLORA_OK) return rc;
-  if (p.t.n_adapters == 0) return SLORA_OK;  // no request can name an adapter
-  if (o == nullptr || x == nullptr || w == nullptr || scales == nullptr) return SLORA_ERR_NULL_POINTER;
-  if (feat_out > (1 << 21) || max_rank > SLORA_MAX_RANK || page_elems > (1LL << 30)) return SLORA_ERR_UNSUPPORTED;
-  p.o = o;
-  p.x = x;
-  p.w = w;
-  p.scales = scales;
-  p.scales_dtype = scales_dtype;
-  p.x_stride = x_row_stride;
-  p.w_stride = w_row_stride;
-  p.o_stride = o_row_stride;
-  p.page_elems = page_elems;
-  p.feat_out = (int)feat_out;
-  p.max_rank = (int)max_rank;
-  p.qkvo = qkvo;
-  p.n_chunks = (int)((feat_out + kExpGroup - 1) / kExpGroup);
-  // rows a workgroup walks: up to kExpSpanTiles tiles, fewer while that leaves the chip short of workgroups
-  int64_t tiles = kExpSpanTiles;
-  while (tiles > 1 &&
-         n_requests * ((max_input_len + kExpTMW * tiles - 1) / (kExpTMW * tiles)) * p.n_chunks < kExpMinGrid)
-    tiles >>= 1;
-  p.m_span = (int)(kExpTMW * tiles);
-  p.row_cap = max_input_len > (1 << 30) ? (1 << 30) : (int)((max_input_len + kExpTMW - 1) / kExpTMW * kExpTMW);
-  p.m_tiles = (int)((max_input_len + p.m_span - 1) / p.m_span);
-  p.vec_ok = (feat_out % 8 == 0) && (page_elems % 8 == 0) && (x_row_stride % 8 == 0) && (w_row_stride % 8 == 0) &&
-             (o_row_stride % 8 == 0) && aligned16(o) && aligned16(x) && aligned16(w);
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  return dtype == SLORA_DTYPE_F16 ? launch_seg_expand<F16>(p, s) : launch_seg_expand<BF16>(p, s);
+  void* const os[3] = {o, nullptr, nullptr};
+  const void* const xs[3] = {x, nullptr, nullptr};
+  const int64_t feats[3] = {feat_out, 0, 0}, o_strides[3] = {o_row_stride, 0, 0};
+  return slora::seg_expand_common(os, xs, 1, w, tables, scales, scales_dtype, b_start_loc, b_seq_len, b_indicies,
+                                  n_requests, max_input_len, n_tokens, feats, page_elems, max_rank, x_row_stride,
+                                  w_row_stride, o_strides, n_pages, qkvo, dtype, stream);
+}
+
+int slora_sgmm_expand_qkv(void* o_q, void* o_k, void* o_v, const void* x_q, const void* x_k, const void* x_v,
+                          const void* w, const slora_tables* tables, const void* scales, int scales_dtype,
+                          const int32_t* b_start_loc, const int32_t* b_seq_len, const int64_t* b_indicies,
+                          int64_t n_requests, int64_t max_input_len, int64_t n_tokens, int64_t feat_out_q,
+                          int64_t feat_out_kv, int64_t page_elems, int64_t max_rank, int64_t x_row_stride,
+                          int64_t w_row_stride, int64_t o_row_stride_q, int64_t o_row_stride_kv, int64_t n_pages,
+                          int dtype, void* stream) {
+  void* const os[3] = {o_q, o_k, o_v};
+  const void* const xs[3] = {x_q, x_k, x_v};
+  const int64_t feats[3] = {feat_out_q, feat_out_kv, feat_out_kv};
+  const int64_t o_strides[3] = {o_row_stride_q, o_row_stride_kv, o_row_stride_kv};
+  return slora::seg_expand_common(os, xs, 3, w, tables, scales, scales_dtype, b_start_loc, b_seq_len, b_indicies,
+                                  n_requests, max_input_len, n_tokens, feats, page_elems, max_rank, x_row_stride,
+                                  w_row_stride, o_strides, n_pages, 0, dtype, stream);
 }
 
 }  // extern "C"

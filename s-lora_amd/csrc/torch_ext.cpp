@@ -749,6 +749,42 @@ void lora_get_qkvo_fwd_expand(const Tensor& x, const Tensor& w, const Tensor& o,
                  " qkvo=" + std::to_string(qkvo) + ")");
 }
 
+// q, k and v expand of one layer in one launch (no counterpart in the reference, which issues the
+// three calls of lora_unordered_batch_infer.py:349-372, 383-398, 409-424): the results are those of the
+// three calls bit for bit.  o_k and o_v share width and row stride (grouped-query models: narrower
+// than o_q); x_q, x_k and x_v share shape and row stride.
+void lora_get_qkvo_fwd_expand_qkv(const Tensor& x_q, const Tensor& x_k, const Tensor& x_v, const Tensor& w,
+                                  const Tensor& o_q, const Tensor& o_k, const Tensor& o_v, const Tensor& scale,
+                                  const Tensor& b_loc, const Tensor& b_lora_start, const Tensor& b_lora_ranks,
+                                  const Tensor& b_start_loc, const Tensor& b_seq_len, const Tensor& b_indicies,
+                                  int64_t feat_out_q, int64_t feat_out_kv, int64_t max_rank, int64_t max_input_len) {
+  const slora_tables t = prefill_common(x_q, w, o_q, b_loc, b_lora_start, b_lora_ranks, b_start_loc, b_seq_len, b_indicies);
+  for (const Tensor* a : {&x_k, &x_v, &o_k, &o_v}) check_2d_strided(*a, "x_k / x_v / o_k / o_v");
+  TORCH_CHECK(x_k.scalar_type() == x_q.scalar_type() && x_v.scalar_type() == x_q.scalar_type() &&
+                  o_k.scalar_type() == x_q.scalar_type() && o_v.scalar_type() == x_q.scalar_type(),
+              "x_q, x_k, x_v, o_q, o_k and o_v must share their dtype");
+  TORCH_CHECK(x_k.sizes() == x_q.sizes() && x_v.sizes() == x_q.sizes() && x_k.stride(0) == x_q.stride(0) &&
+                  x_v.stride(0) == x_q.stride(0),
+              "x_q, x_k and x_v must share shape and row stride");
+  TORCH_CHECK(o_k.sizes() == o_v.sizes() && o_k.stride(0) == o_v.stride(0) && o_k.size(0) == o_q.size(0),
+              "o_k and o_v must share shape and row stride, and have as many rows as o_q");
+  TORCH_CHECK(scale.is_cuda() && scale.is_contiguous(), "scale must be a contiguous CUDA tensor");
+  const int sc = dtype_code(scale, "scale");
+  TORCH_CHECK(scale.numel() >= b_lora_start.numel(), "scale must have one entry per adapter");
+  TORCH_CHECK(o_q.size(1) >= feat_out_q && o_k.size(1) >= feat_out_kv && x_q.size(1) >= max_rank,
+              "o narrower than feat_out or x narrower than max_rank");
+  const int rc = slora_sgmm_expand_qkv(o_q.data_ptr(), o_k.data_ptr(), o_v.data_ptr(), x_q.data_ptr(), x_k.data_ptr(),
+                                       x_v.data_ptr(), w.data_ptr(), &t, scale.data_ptr(), sc,
+                                       b_start_loc.data_ptr<int32_t>(), b_seq_len.data_ptr<int32_t>(),
+                                       b_indicies.data_ptr<int64_t>(), b_seq_len.numel(), max_input_len, x_q.size(0),
+                                       feat_out_q, feat_out_kv, w.size(1), max_rank, x_q.stride(0), w.stride(0),
+                                       o_q.stride(0), o_k.stride(0), w.size(0), dtype_code(x_q, "x"), stream_of(x_q));
+  if (rc != SLORA_OK)
+    check_rc(rc, "lora_get_qkvo_fwd_expand_qkv",
+             "(feat_out_q=" + std::to_string(feat_out_q) + " feat_out_kv=" + std::to_string(feat_out_kv) +
+                 " max_rank=" + std::to_string(max_rank) + ")");
+}
+
 // ---------------------------------------------------------------------------
 // pool helpers (slora/server/router/model_infer/infer_adapter.py, slora/common/mem_allocator.py)
 // ---------------------------------------------------------------------------
@@ -1005,6 +1041,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("lora_get_qkvo_fwd_expand", &lora_get_qkvo_fwd_expand, py::arg("x"), py::arg("w"), py::arg("o"), py::arg("scale"),
         py::arg("b_loc"), py::arg("b_lora_start"), py::arg("b_lora_ranks"), py::arg("b_start_loc"), py::arg("b_seq_len"),
         py::arg("b_indicies"), py::arg("feat_out"), py::arg("qkvo"), py::arg("max_rank"), py::arg("max_input_len"));
+  m.def("lora_get_qkvo_fwd_expand_qkv", &lora_get_qkvo_fwd_expand_qkv, py::arg("x_q"), py::arg("x_k"), py::arg("x_v"),
+        py::arg("w"), py::arg("o_q"), py::arg("o_k"), py::arg("o_v"), py::arg("scale"), py::arg("b_loc"),
+        py::arg("b_lora_start"), py::arg("b_lora_ranks"), py::arg("b_start_loc"), py::arg("b_seq_len"),
+        py::arg("b_indicies"), py::arg("feat_out_q"), py::arg("feat_out_kv"), py::arg("max_rank"),
+        py::arg("max_input_len"));
   m.def("make_prefill_plan", &make_prefill_plan, py::arg("b_lora_start"), py::arg("b_lora_ranks"), py::arg("b_start_loc"),
         py::arg("b_seq_len"), py::arg("b_indicies"), py::arg("n_tokens"), py::arg("max_rank"), py::arg("max_input_len"));
 

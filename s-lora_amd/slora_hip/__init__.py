@@ -30,7 +30,8 @@ except ImportError as e:  # pragma: no cover
 
 from ._kernels import (BgmvPlan, SgmmPlan, clear_plan_cache, clear_prefill_plan_cache,  # noqa: F401,E402
                        dispatch_bgmv, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_shrink,
-                       lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv, make_plan,
+                       lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_expand_qkv, lora_get_qkvo_fwd_shrink,
+                       lora_get_qkvo_fwd_shrink_qkv, make_plan,
                        make_prefill_plan, plan_cache_stats, rebuild_plan, set_plan_cache_enabled)
 from .lora_unordered_batch_infer import LoraUnorderedBatchInfer  # noqa: F401,E402
 

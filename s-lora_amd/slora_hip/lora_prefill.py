@@ -15,6 +15,10 @@ from ``make_prefill_plan`` for this batch (same results; the split of the batch
 over the workgroups is read instead of recomputed).  Without it the plan of the
 last call with the same five index tensors is reused; ``plan=False`` forces the
 kernel that needs no plan.
+
+``lora_get_qkvo_fwd_shrink_qkv`` and ``lora_get_qkvo_fwd_expand_qkv`` do the q, k and v
+calls of a layer in one launch each (same bits as the three calls).
 """
 from ._kernels import (SgmmPlan, clear_prefill_plan_cache, lora_get_qkvo_fwd_expand,  # noqa: F401
-                       lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv, make_prefill_plan)
+                       lora_get_qkvo_fwd_expand_qkv, lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv,
+                       make_prefill_plan)

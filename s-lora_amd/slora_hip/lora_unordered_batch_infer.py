@@ -15,9 +15,8 @@ Two ways to issue the work, same results bit for bit:
 * ``fused=False``: the reference's call sequence, one ``dispatch_bgmv`` or
   ``lora_get_qkvo_fwd_*`` call per projection and direction (8 per layer),
   ``delta[0]`` shared by q and o as in the reference;
-* ``fused=True`` (default): q, k and v of a layer in one shrink launch and one
-  expand launch (decode), or one shrink launch that reads the activations once
-  (prefill).
+* ``fused=True`` (default): q, k and v of a layer in one shrink launch (which reads
+  the activations once) and one expand launch, in decode and in prefill steps.
 
 Either way the first call of a step builds the batch's plan inside the library and
 the other calls of the step reuse it (the index tensors are the same objects in
@@ -30,7 +29,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from ._kernels import (dispatch_bgmv, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_shrink, lora_get_qkvo_fwd_expand,
-                       lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv)
+                       lora_get_qkvo_fwd_expand_qkv, lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv)
 
 # lora_unordered_batch_infer.py:334: the segmented kernels serve batches with a long
 # request, adapters of rank >= 64 and at least two requests; everything else is BGMV
@@ -129,6 +128,11 @@ class LoraUnorderedBatchInfer:
                 for p in range(3):
                     lora_get_qkvo_fwd_shrink(input_embs, key2, d[p], *seg, hidden, p, self.max_lora_dim,
                                              self.max_b_seq_len)
+            if self.fused and cache_k.shape == cache_v.shape and cache_k.stride(0) == cache_v.stride(0):
+                lora_get_qkvo_fwd_expand_qkv(d[0], d[1], d[2], val2, q, cache_k, cache_v, ia.a_scaling, *seg,
+                                             int(q.shape[1]), int(cache_k.shape[1]), self.max_lora_dim,
+                                             self.max_b_seq_len)
+                return
             for p in range(3):
                 lora_get_qkvo_fwd_expand(d[p], val2, outs[p], ia.a_scaling, *seg, int(outs[p].shape[1]), p,
                                          self.max_lora_dim, self.max_b_seq_len)

@@ -55,6 +55,8 @@ SIGNATURES = {
                                    _I64, _I64, _I, _P]),
     "slora_sgmm_expand": (_I, [_P, _P, _P, _TP, _P, _I, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I64, _I64, _I, _I, _P]),
+    "slora_sgmm_expand_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _TP, _P, _I, _P, _P, _P, _I64, _I64, _I64, _I64, _I64,
+                                   _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I, _P]),
     "slora_pool_scatter_rows": (_I, [_P, _P, _I, _P, _I64, _I64, _I64, _I64, _I64, _P]),
     "slora_pool_pack_transposed": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I64, _I64, _I64, _P]),
     "slora_var_len_copy": (_I, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _P]),

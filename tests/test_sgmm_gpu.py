@@ -409,3 +409,63 @@ def test_prefill_qkv_shrink_rejects_mismatched_outputs(gpu):
     with pytest.raises(RuntimeError, match="share dtype, shape and row stride"):
         lora_get_qkvo_fwd_shrink_qkv(g.x, g.key.view(c.n_pages, c.page_elems), o[0], o[1], wide, g.a_loc, g.a_start,
                                      g.a_len, start, lens, ids, c.hidden, 16, max_len)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,h_kv,ranks,n_req,lo,hi", [
+    (512, 512, [64, 8, 16, 32], 9, 1, 120),        # q, k and v as wide as a page
+    (1024, 256, [64, 16], 6, 8, 200),              # grouped-query widths: k and v a quarter of a page
+    (512, 128, [8, 32], 5, 1, 40),                 # k and v narrower than one output group of a workgroup
+    (256, 256, [16, 32], 300, 1, 9),               # more requests than one workgroup describes
+    (256, 256, [12, 8, 20], 5, 3, 40),             # ranks that take the element-wise path
+    (4096, 4096, [64, 32, 16, 8], 12, 100, 600),   # C3's widths
+])
+def test_prefill_qkv_expand_gives_the_three_calls_bits(gpu, dtype, hidden, h_kv, ranks, n_req, lo, hi):
+    """lora_get_qkvo_fwd_expand_qkv (one launch for q, k and v) against the three calls the reference
+    issues (lora_unordered_batch_infer.py:349-372 and the k, v blocks after it): identical bits,
+    also in rows that belong to no request and in the columns beyond the outputs' widths; one of
+    the three results is checked against the oracle."""
+    from slora_hip import lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_expand_qkv
+    c = seg_case(2300 + hidden + n_req, hidden, ranks, n_req, lo, hi, dtype, h_out=[hidden, h_kv, h_kv, hidden])
+    g = GpuCase(c, gpu)
+    start, lens, ids = dev(c.start, torch.int32, gpu), dev(c.lens, torch.int32, gpu), dev(c.ids, torch.int64, gpu)
+    max_len = int(c.lens.max())
+    R = (max(ranks) + 7) // 8 * 8
+    T = c.batch
+    rng = np.random.default_rng(5)
+    w_b = g.value.view(c.n_pages, c.page_elems)
+    t = (g.a_loc, g.a_start, g.a_len, start, lens, ids)
+    widths = [hidden, h_kv, h_kv]
+    deltas = [dev(O.round_to(rng.standard_normal((T + 2, R)).astype(np.float32), c.dtype), g.tdt, gpu) for _ in range(3)]
+    y0 = [O.round_to(rng.standard_normal((T + 2, widths[p] + 8)).astype(np.float32), c.dtype) for p in range(3)]
+    single = [dev(y0[p], g.tdt, gpu) for p in range(3)]
+    for p in range(3):
+        lora_get_qkvo_fwd_expand(deltas[p], w_b, single[p][:, :widths[p]], g.scales, *t, widths[p], p, R, max_len)
+    fused = [dev(y0[p], g.tdt, gpu) for p in range(3)]
+    lora_get_qkvo_fwd_expand_qkv(deltas[0], deltas[1], deltas[2], w_b, fused[0][:, :hidden], fused[1][:, :h_kv],
+                                 fused[2][:, :h_kv], g.scales, *t, hidden, h_kv, R, max_len)
+    torch.cuda.synchronize()
+    for p in range(3):
+        assert torch.equal(fused[p], single[p]), p
+        assert torch.equal(fused[p][T:], dev(y0[p], g.tdt, gpu)[T:])           # rows of no request
+        assert torch.equal(fused[p][:, widths[p]:], dev(y0[p], g.tdt, gpu)[:, widths[p]:])
+    y_ref = O.ref_prefill_expand(y0[2][:T, :h_kv], host(deltas[2])[:T], c.value, c.scales, c.a_loc, c.a_start, c.a_len,
+                                 c.start, c.lens, c.ids, 2, R, c.dtype)
+    np.testing.assert_allclose(host(fused[2][:T, :h_kv]), y_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_prefill_qkv_expand_rejects_mismatched_tensors(gpu):
+    from slora_hip import lora_get_qkvo_fwd_expand_qkv
+    c = seg_case(34, 256, [16, 8], 6, 1, 50, "f16")
+    g = GpuCase(c, gpu)
+    start, lens, ids = dev(c.start, torch.int32, gpu), dev(c.lens, torch.int32, gpu), dev(c.ids, torch.int64, gpu)
+    d = [torch.zeros((c.batch, 16), dtype=g.tdt, device=gpu) for _ in range(3)]
+    y = [torch.zeros((c.batch, 256), dtype=g.tdt, device=gpu) for _ in range(2)]
+    narrow = torch.zeros((c.batch, 128), dtype=g.tdt, device=gpu)
+    t = (g.a_loc, g.a_start, g.a_len, start, lens, ids)
+    with pytest.raises(RuntimeError, match="o_k and o_v must share shape"):
+        lora_get_qkvo_fwd_expand_qkv(d[0], d[1], d[2], g.value.view(c.n_pages, 256), y[0], y[1], narrow, g.scales, *t,
+                                     256, 256, 16, int(c.lens.max()))
+    with pytest.raises(RuntimeError, match="x_q, x_k and x_v must share shape"):
+        lora_get_qkvo_fwd_expand_qkv(d[0], d[1], d[2][:, :8], g.value.view(c.n_pages, 256), y[0], y[1], y[1], g.scales,
+                                     *t, 256, 256, 16, int(c.lens.max()))
