@@ -80,18 +80,21 @@ class LoraUnorderedBatchInfer:
 
     # ---- per step (forward(), :44-80) -----------------------------------------------------
     def begin_step(self, b_start_loc: torch.Tensor, b_seq_len: torch.Tensor, is_prefill: bool,
-                   max_b_seq_len: Optional[int] = None) -> None:
+                   max_b_seq_len: Optional[int] = None, total_token_num: Optional[int] = None) -> None:
         """The per-step part of ``forward``: ``delta`` (three zeroed ``[tokens, max_lora_dim]``
         buffers, :69 / :76), per-token adapter ids for a prefill batch (:66) and the kernel choice
         (:334).  ``max_b_seq_len`` spares the read-back of ``torch.max(b_seq_len).item()`` (:61)
-        when the caller knows it."""
+        and ``total_token_num`` (the sum of ``b_seq_len``, an argument of the reference's ``forward``)
+        the one inside ``repeat_interleave``, when the caller knows them: the step then starts
+        without waiting for the device."""
         assert b_start_loc.shape[0] == b_seq_len.shape[0] == self.req_bins.shape[0]
         self.is_prefill = bool(is_prefill)
         self.b_start_loc, self.b_seq_len = b_start_loc, b_seq_len
         self.max_b_seq_len = int(max_b_seq_len) if max_b_seq_len is not None else int(torch.max(b_seq_len).item())
         n_req = int(b_seq_len.shape[0])
         if self.is_prefill:
-            self.batch_req_bins = torch.repeat_interleave(self.req_bins, b_seq_len.to(torch.long))
+            self.batch_req_bins = torch.repeat_interleave(self.req_bins, b_seq_len.to(torch.long),
+                                                          output_size=total_token_num)
             n_tok = int(self.batch_req_bins.shape[0])
             self.use_segmented = (self.max_b_seq_len >= PREFILL_MIN_SEQ_LEN and
                                   self.max_lora_dim >= PREFILL_MIN_LORA_DIM and n_req >= PREFILL_MIN_REQUESTS)

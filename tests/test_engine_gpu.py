@@ -144,7 +144,11 @@ def test_prefill_step_kernel_choice_and_results(gpu, lens, segmented):
     res = {}
     for fused in (True, False):
         eng = LoraUnorderedBatchInfer(m.ia, [m.adapters[n] for n in req], fused=fused)
-        eng.begin_step(b_start, b_seq_len, is_prefill=True)      # reads max(b_seq_len) back, as the reference does
+        if fused:     # reads max(b_seq_len) and the token count back, as the reference does
+            eng.begin_step(b_start, b_seq_len, is_prefill=True)
+        else:         # or is told both
+            eng.begin_step(b_start, b_seq_len, is_prefill=True, max_b_seq_len=int(lens_np.max()),
+                           total_token_num=int(lens_np.sum()))
         assert eng.use_segmented == segmented and eng.max_b_seq_len == int(lens_np.max())
         assert eng.batch_req_bins.cpu().tolist() == bins.tolist()
         res[fused] = _run_layers(m, eng, gpu, x, base)
