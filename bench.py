@@ -661,6 +661,20 @@ def main():
         return max(ev_ms, wall_ms) if args.launch == "direct" else ev_ms
 
     ms_per_step = time_steps(run_step)
+
+    def step_percentiles(fn, reps=100):
+        """every step between its own pair of events: spread of the step time (not part of `value`)"""
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for a, b in evs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        return {"reps": reps, "p10": round(ts[reps // 10], 4), "median": round(ts[reps // 2], 4),
+                "p90": round(ts[reps * 9 // 10], 4)}
+
+    spread = step_percentiles(run_step) if use_graph else None
     other_modes = {}
     if args.all_modes:
         for m in ("dropin", "fused", "planned", "planned-fused"):
@@ -723,6 +737,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
+        "step_ms_spread": spread,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
