@@ -98,6 +98,16 @@ def test_sgmm_argument_checks(lib):
     assert e(P, P, P, C.byref(t), P, A.DTYPE_F16, P, P, P, 0, 0, 0, 4096, 4096, 64, 64, 4096, 4096, 100, 0, A.DTYPE_F16, None) == A.OK
     assert e(P, P, P, C.byref(t), None, A.DTYPE_F16, P, P, P, 4, 16, 64, 4096, 4096, 64, 64, 4096, 4096, 100, 0, A.DTYPE_F16, None) == A.ERR_NULL_POINTER
     assert e(P, P, P, C.byref(t), P, A.DTYPE_F16, P, P, P, 4, 16, 64, 4096, 4096, 64, 32, 4096, 4096, 100, 0, A.DTYPE_F16, None) == A.ERR_BAD_SHAPE
+    # q, k and v in one launch: o_q o_k o_v x_q x_k x_v w tables scales scales_dtype b_start_loc b_seq_len b_indicies
+    # n_requests max_input_len n_tokens feat_out_q feat_out_kv page_elems max_rank x_stride w_stride o_stride_q o_stride_kv n_pages dtype stream
+    f = lib.slora_sgmm_expand_qkv
+    head = (P, P, P, P, P, P, P, C.byref(t), P, A.DTYPE_F16, P, P, P)
+    assert f(*head, 0, 0, 0, 4096, 1024, 4096, 64, 64, 4096, 4096, 1024, 100, A.DTYPE_F16, None) == A.OK
+    assert f(*head, 4, 16, 64, 4096, 1024, 4096, 64, 64, 4096, 4096, 512, 100, A.DTYPE_F16, None) == A.ERR_BAD_SHAPE   # o_k rows narrower than feat_out_kv
+    assert f(*head, 4, 16, 64, 4096, 1024, 4096, 64, 32, 4096, 4096, 1024, 100, A.DTYPE_F16, None) == A.ERR_BAD_SHAPE  # x rows narrower than max_rank
+    assert f(*head, 4, 16, 64, 4096, 1024, 4096, 64, 64, 4096, 4096, 1024, 100, 9, None) == A.ERR_BAD_DTYPE
+    assert f(P, None, P, P, P, P, P, C.byref(t), P, A.DTYPE_F16, P, P, P, 4, 16, 64, 4096, 1024, 4096, 64, 64, 4096, 4096,
+             1024, 100, A.DTYPE_F16, None) == A.ERR_NULL_POINTER
 
 
 def test_python_mirror_rejects_cpu_tensors():
