@@ -367,6 +367,10 @@ def test_prefill_plan_of_another_batch_is_rejected(gpu):
     (200, [8, 40, 16], 7, 1, 90, False),           # hidden size that is no multiple of 64: ragged last k block
     (64, [8], 3, 1, 20, True),                     # a single k block per row
     (128, [16, 8], 4, 1, 30, True),                # two k blocks: fewer blocks than wavefronts
+    # larger batches (more row parts than workgroups of a launch)
+    (256, [16, 8, 64, 32], 45, 90, 130, True),
+    (200, [8, 40, 16], 50, 80, 120, False),        # ragged last k block, a rank on the element-wise path
+    (320, [128, 24], 300, 10, 22, False),          # two passes over the rank, more requests than a plan describes
 ])
 def test_prefill_qkv_shrink_gives_the_three_calls_bits(gpu, dtype, hidden, ranks, n_req, lo, hi, sort):
     """lora_get_qkvo_fwd_shrink_qkv (x read once for q, k and v) against the three calls
