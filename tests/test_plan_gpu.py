@@ -60,6 +60,7 @@ def expected_plan(bins, a_start, a_len, a_loc, n_pages, rank_cap):
     (64, 5, 16, 4),                                                            # ranks above the cap: `more`
     (1025, 200, 64, 5), (3000, 1500, 32, 6), (8192, 64, 64, 7), (5000, 5000, 8, 8),   # sorted in LDS
     (9000, 300, 64, 9),                                                        # one workgroup
+    (2000, 600000, 64, 10),                                                    # adapter ids too large for the sorted keys
 ])
 def test_plan_records_word_for_word(gpu, batch, n_adapters, rank_cap, seed):
     import slora_hip
@@ -67,14 +68,23 @@ def test_plan_records_word_for_word(gpu, batch, n_adapters, rank_cap, seed):
     ranks = rng.choice([8, 16, 32, 64, 24, 0], size=n_adapters, p=[.25, .2, .2, .2, .1, .05])
     if seed == 4:
         ranks = np.array([64, 8, 32, 128, 16])
+    if n_adapters > 100000:       # a few adapters with weights among many without
+        live = rng.choice(n_adapters, size=80, replace=False)
+        keep = ranks[live]
+        ranks = np.zeros(n_adapters, dtype=ranks.dtype)
+        ranks[live] = keep
     a_len = (4 * ranks).astype(np.int64)
     a_start = np.concatenate([[0], np.cumsum(a_len)[:-1]]).astype(np.int64)
     n_loc = int(a_len.sum())
     n_pages = n_loc + 50
     a_loc = rng.permutation(n_pages)[:n_loc].astype(np.int64)
     a_loc[rng.integers(0, max(n_loc, 1), size=3)] = n_pages + 7          # page ids outside the pool
-    p = 1.0 / np.arange(1, n_adapters + 1)
-    bins = rng.choice(n_adapters, size=batch, p=p / p.sum()).astype(np.int64)
+    if n_adapters > 100000:
+        pool_ids = np.concatenate([np.nonzero(ranks)[0], rng.integers(0, n_adapters, size=20)])
+        bins = rng.choice(pool_ids, size=batch).astype(np.int64)
+    else:
+        p = 1.0 / np.arange(1, n_adapters + 1)
+        bins = rng.choice(n_adapters, size=batch, p=p / p.sum()).astype(np.int64)
     bins[rng.integers(0, batch, size=max(1, batch // 50))] = -1           # tokens without an adapter
     bins[rng.integers(0, batch, size=max(1, batch // 70))] = n_adapters + 3
     t = [torch.from_numpy(v).to(gpu) for v in (a_start, a_len, a_loc, bins)]
