@@ -320,18 +320,31 @@ class InferAdapter:
         self.a_scaling = torch.cat((self.a_scaling, torch.tensor([a.scaling for a in new_adapters],
                                                                  dtype=torch.float16, device=dev)))
 
-        def copy_all():
+        def copy_all(loc):
             cum = 0
             for a, n in zip(new_adapters, lens):
-                self._load_weights(a, new_loc[cum: cum + n])
+                self._load_weights(a, loc[cum: cum + n])
                 cum += n
 
         if prefetch and self.prefetch_stream is not None:
-            self.prefetch_stream.wait_stream(torch.cuda.current_stream())  # new_loc is produced on this stream
-            with torch.cuda.stream(self.prefetch_stream):
-                copy_all()
+            side = self.prefetch_stream
+            side.wait_stream(torch.cuda.current_stream())  # new_loc is produced on this stream
+            with torch.cuda.stream(side):
+                # the page list the loaders read is the side stream's own copy (as the reference's clone,
+                # :153-155): new_loc goes out of scope when this function returns, and a block that the main
+                # stream's allocator hands out again must not be one the queued kernels still read
+                loc_side = new_loc.clone()
+                new_loc.record_stream(side)
+                for a in new_adapters:
+                    # weights produced on the main stream and read by kernels queued on the side stream
+                    for name in ("lora_A", "lora_B"):
+                        for per_layer in getattr(a, name, None) or ():
+                            for m in (per_layer if isinstance(per_layer, (list, tuple)) else (per_layer,)):
+                                if torch.is_tensor(m) and m.is_cuda:
+                                    m.record_stream(side)
+                copy_all(loc_side)
         else:
-            copy_all()
+            copy_all(new_loc)
 
     def offload_adapters(self, reserve_adapter_dirs) -> None:
         if len(reserve_adapter_dirs) == len(self.adapter_dirs):

@@ -221,16 +221,18 @@ def test_decode_and_prefill_match_ref_bmm(gpu, plan_cache_mode, dtype, hidden, r
     shrink output (``ref_bmm`` with x = delta and A = the identity, whose ``x @ A`` is delta
     exactly), from a zero y.
 
-    The whole chain shrink -> expand against ``ref_bmm(x, A, B)``: rtol 1e-2 and an absolute
-    term of 1e-3 plus what ONE storage-type rounding flip per delta entry moves y by,
-    ``ulp(max|delta_t|) * scale * sum_d |B[d, n]|``.  The intermediate delta is rounded to
+    The whole chain shrink -> expand against ``ref_bmm(x, A, B)``: rtol 1e-2 / atol 1e-3 for
+    every output but a counted few -- at most 1 in 10 000 may lie outside, and then by no more
+    than what ONE storage-type rounding flip of ONE delta entry moves that output by,
+    ``ulp(max|delta_t|) * scale * max_d |B[d, n]|``.  The intermediate delta is rounded to
     fp16/bf16 by the engine and by the kernels alike, from float sums taken in different
     orders; where a sum lies within a float ulp of a rounding boundary the two round apart,
-    and y, a sum of r such entries times B of order 1/sqrt(r), moves by that much whatever
-    the kernel does.  (Measured: 5 of 131072 outputs of the C1 case differ by up to 2e-3
-    where y is near zero.)  From a random y the absolute term also holds one ulp of the sum
-    y0 + update (|.| < 16: 2^-7 in fp16, 2^-4 in bf16), the rounding ``+=`` has in the
-    reference itself."""
+    whatever the kernel does.  (Measured: 5 of 131072 outputs of the C1 case differ by up to
+    2e-3 where y is near zero.)  From a random y every output is also allowed one rounding
+    step of the storage type at the magnitude of the larger operand of ``y0 + update``: the
+    reference's ``+=`` rounds the update (product, then times scaling) and the sum at that
+    magnitude, the kernels round scale * sum once, and where y0 and the update cancel that
+    step is larger than any tolerance relative to the small result."""
     from slora_hip import dispatch_bgmv, lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_shrink
     n_ad = len(ranks)
     rng = np.random.default_rng(3)
@@ -250,7 +252,6 @@ def test_decode_and_prefill_match_ref_bmm(gpu, plan_cache_mode, dtype, hidden, r
     t = (g.a_start, g.a_len, g.a_loc, g.bins)
     tp = (g.a_loc, g.a_start, g.a_len, st, ln, rq)
     mant = 10 if dtype == "f16" else 7
-    ulp_sum = 2.0 ** (4 - 1 - mant)
     eye = [np.eye(R, r, dtype=np.float32) for r in ranks]
     for p in range(4):
         A_p, B_p = [a[p] for a in c.A], [b[p] for b in c.B]
@@ -260,15 +261,20 @@ def test_decode_and_prefill_match_ref_bmm(gpu, plan_cache_mode, dtype, hidden, r
         for tkn in range(batch):
             a = c.bins[tkn]
             xa[tkn, : ranks[a]] = O.round_to(c.x[tkn] @ A_p[a], dtype)
-        # per output: what one rounding flip of every delta entry of the token can move it by
+        # per output: what one rounding flip of one delta entry of the token can move it by
         ulp_d = 2.0 ** (np.floor(np.log2(np.abs(xa).max(axis=1) + 1e-30)) - mant)
-        flip = np.stack([ulp_d[tkn] * c.scales[c.bins[tkn]] * np.abs(B_p[c.bins[tkn]]).sum(axis=0)
+        flip = np.stack([ulp_d[tkn] * c.scales[c.bins[tkn]] * np.abs(B_p[c.bins[tkn]]).max(axis=0)
                          for tkn in range(batch)])
 
-        def close(got, want, atol_extra=0.0):
+        def close(got, want, start=None):
             err = np.abs(got - want)
-            tol = RTOL * np.abs(want) + ATOL + atol_extra
-            assert np.all(err <= tol), (p, float((err - tol).max()), int((err > tol).sum()))
+            tol = RTOL * np.abs(want) + ATOL
+            if start is not None:   # one step of the storage type at the magnitude of y0 or of the update
+                big = np.maximum(np.abs(start), np.abs(want - start))
+                tol = tol + 2.0 ** (np.floor(np.log2(big + 1e-30)) - mant)
+            bad = err > tol
+            assert bad.sum() <= max(1, int(1e-4 * bad.size)), (p, int(bad.sum()), bad.size, float((err - tol).max()))
+            assert np.all(err[bad] <= tol[bad] + flip[bad]), (p, float((err - tol - flip)[bad].max()))
 
         # ---- decode
         d = torch.zeros((batch, R), dtype=g.tdt, device=gpu)
@@ -278,10 +284,10 @@ def test_decode_and_prefill_match_ref_bmm(gpu, plan_cache_mode, dtype, hidden, r
         dispatch_bgmv(y, d, g.value, *t, p, g.scales)
         np.testing.assert_allclose(host(y), O.ref_bmm(zero, host(d), eye, B_p, c.scales, c.bins, dtype),
                                    rtol=RTOL, atol=ATOL)
-        close(host(y), O.ref_bmm(zero, c.x, A_p, B_p, c.scales, c.bins, dtype), flip)
+        close(host(y), O.ref_bmm(zero, c.x, A_p, B_p, c.scales, c.bins, dtype))
         y = dev(y0, g.tdt, gpu)
         dispatch_bgmv(y, d, g.value, *t, p, g.scales)
-        close(host(y), O.ref_bmm(y0, c.x, A_p, B_p, c.scales, c.bins, dtype), flip + ulp_sum)
+        close(host(y), O.ref_bmm(y0, c.x, A_p, B_p, c.scales, c.bins, dtype), y0)
         # ---- prefill
         o = torch.zeros((batch, R), dtype=g.tdt, device=gpu)
         lora_get_qkvo_fwd_shrink(g.x, g.key.view(c.n_pages, hidden), o, *tp, hidden, p, R, int(lens.max()))
@@ -290,10 +296,10 @@ def test_decode_and_prefill_match_ref_bmm(gpu, plan_cache_mode, dtype, hidden, r
         lora_get_qkvo_fwd_expand(o, g.value.view(c.n_pages, hidden), y2, g.scales, *tp, hidden, p, R, int(lens.max()))
         np.testing.assert_allclose(host(y2), O.ref_bmm(zero, host(o), eye, B_p, c.scales, c.bins, dtype),
                                    rtol=RTOL, atol=ATOL)
-        close(host(y2), O.ref_bmm(zero, c.x, A_p, B_p, c.scales, c.bins, dtype), flip)
+        close(host(y2), O.ref_bmm(zero, c.x, A_p, B_p, c.scales, c.bins, dtype))
         y2 = dev(y0, g.tdt, gpu)
         lora_get_qkvo_fwd_expand(o, g.value.view(c.n_pages, hidden), y2, g.scales, *tp, hidden, p, R, int(lens.max()))
-        close(host(y2), O.ref_bmm(y0, c.x, A_p, B_p, c.scales, c.bins, dtype), flip + ulp_sum)
+        close(host(y2), O.ref_bmm(y0, c.x, A_p, B_p, c.scales, c.bins, dtype), y0)
 
 
 # ---------------------------------------------------------------------------

@@ -402,6 +402,46 @@ def test_infer_adapter_load_offload_and_decode(gpu, placement):
     assert mm.can_use_mem_size == 600 - 25
 
 
+def test_prefetch_keeps_its_page_list_while_the_main_stream_allocates(gpu):
+    """A prefetching load queues its pack kernels on the side stream and returns; the page list
+    they read must stay theirs.  The side stream is kept busy first so that the kernels are still
+    queued when the main stream allocates and overwrites int64 tensors of the page list's size
+    (what the caching allocator would hand out if the list's block had been given back): every
+    page must still hold the packed weights, bit for bit."""
+    from slora_hip.infer_adapter import InferAdapter, MemoryAllocator, page_checksums
+    H, L, heads, r = 256, 2, 4, 16
+    rng = np.random.default_rng(11)
+    mm = MemoryAllocator(400, 0, torch.float16, heads, H // heads, L, device=gpu)
+    for b in mm.key_buffer + mm.value_buffer:
+        b.zero_()
+    side = torch.cuda.Stream()
+    ia = InferAdapter.init(mm, prefetch_stream=side, device=gpu)
+    A, B = _np_mats(rng, H, [H] * 4, r, L, "f16")
+    ad = _Adapter("p", r, 16.0, [[torch.from_numpy(a).to(gpu, torch.float16) for a in A[l]] for l in range(L)],
+                  [[torch.from_numpy(b).to(gpu, torch.float16) for b in B[l]] for l in range(L)])
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(50_000_000)        # tens of milliseconds: the loads below queue behind it
+    ia.load_adapters([ad], prefetch=True)
+    junk = []
+    for _ in range(64):                       # same size and dtype as the page list: the same allocator bin
+        t = torch.empty(4 * r, dtype=torch.int64, device=gpu)
+        t.fill_(399)                          # a valid page nobody owns
+        junk.append(t)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    loc = ia.a_loc.cpu().numpy()
+    assert np.array_equal(loc, np.arange(4 * r))          # first free pages of an empty map
+    for l in range(L):
+        w = O.pack_w_combined(A[l], B[l], H)               # [2, 4r, H]
+        for side_i, buf in ((0, mm.key_buffer[l]), (1, mm.value_buffer[l])):
+            want = O.round_to(w[side_i], "f16").astype(np.float16).view(np.uint32)
+            got = page_checksums(buf, ia.a_loc).cpu().numpy().view(np.uint32)
+            assert np.array_equal(got, np.bitwise_xor.reduce(want, axis=1)), (l, side_i)
+            assert int(page_checksums(buf, torch.tensor([399], device=gpu)).item()) == 0
+    assert len(junk) == 64
+
+
 def test_memory_allocator_places_an_adapter_in_one_run(gpu):
     """alloc_adapter: one contiguous stretch when the map has one (the first such), the first
     free pages otherwise -- against the oracle's alloc_contiguous / alloc."""
