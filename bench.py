@@ -286,6 +286,39 @@ def cpu_baseline(w, bufs, torch, reps_arg):
     }
 
 
+def cpu_baseline_c1(torch):
+    """Configuration 1 exactly: the reference's bmm path on the host cores, float32, hidden 4096,
+    8 adapters of rank 8, 32 tokens with adapter ids uniform in [0, 8), x ~ N(0,1),
+    A ~ N(0, 1/4096), B ~ N(0, 1/8), scaling 2.0, one layer of q/k/v/o."""
+    import numpy as np
+    from oracle import lora_oracle as O
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    rng = np.random.default_rng(1)
+    H, r, n_ad, batch = 4096, 8, 8, 32
+    A = [[(rng.standard_normal((H, r)) / np.sqrt(H)).astype(np.float32) for _ in range(4)] for _ in range(n_ad)]
+    B = [[(rng.standard_normal((r, H)) / np.sqrt(r)).astype(np.float32) for _ in range(4)] for _ in range(n_ad)]
+    bins = rng.integers(0, n_ad, size=batch)
+    layer = O.BmmCpuLayer(A, B, [2.0] * n_ad, bins, threads=threads)
+    x_in = torch.from_numpy(rng.standard_normal((batch, H)).astype(np.float32))
+    x_att = torch.from_numpy(rng.standard_normal((batch, H)).astype(np.float32))
+    ys = [torch.zeros((batch, H), dtype=torch.float32) for _ in range(4)]
+    for _ in range(5):
+        layer.decode(x_in, x_att, ys)
+    times = []
+    for _ in range(30):
+        t0 = time.perf_counter()
+        layer.decode(x_in, x_att, ys)
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    # algorithmic bytes of the layer with 4-byte elements: distinct adapters' A and B, x, delta, y read + written
+    u = np.unique(bins).size
+    nbytes = 4 * (u * r * H * 4 + batch * H * 4 + batch * r * 4) + 4 * (u * r * H * 4 + batch * r * 4 + 2 * batch * H * 4)
+    return {"value": round(batch / med, 1), "unit": "tokens/s per layer", "cores": threads, "kind": "port",
+            "sample": f"one layer of q/k/v/o, fp32, {n_ad} adapters of rank {r}, batch {batch}, median of 30 reps = "
+                      f"{med * 1e3:.3f} ms/layer (5 warm-up)",
+            "gbps_algorithmic": round(nbytes / med / 1e9, 2)}
+
+
 MFMA_PEAK_TFLOPS = 2500.0
 
 
@@ -369,14 +402,16 @@ def measure_other_shapes(w, bufs, torch):
     import subprocess
     free_workload(w, bufs, torch)
     res = {}
-    for wl, layers in (("s4", 8), ("s6", 4)):
+    for wl, layers in (("s4", 8), ("s6", 8)):
         cmd = [sys.executable, os.path.abspath(__file__), "--workload", wl, "--layers", str(layers), "--steps", "10",
                "--warmup", "3", "--no-cpu-baseline", "--no-extras"]
         try:
-            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=240)
+            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True, timeout=300)
             d = json.loads([l for l in proc.stdout.splitlines() if l.startswith("{")][-1])
             res[wl] = {"workload": d["config"]["workload"], "layers": d["config"]["layers"],
                        "ms_per_step": d["ms_per_step"], "tokens_per_s": d["value"], "step_hbm": d["step_hbm"],
+                       "pool_GB": round(2 * d["config"]["layers"] * d["config"]["pool_pages_per_layer"] *
+                                        d["config"]["page_bytes"] / 1e9, 1),
                        "kernels": {k: {"us_per_launch": v["us_per_launch"], "frac": v["frac"],
                                        "kernel_over_ceiling": v.get("read_only_ceiling", {}).get("kernel_over_ceiling")}
                                    for k, v in d["kernels"].items()}}
@@ -484,6 +519,44 @@ def measure_prefill(args, torch, device, w=None, seg=None):
                           "TFLOPs": round(flops / us / 1e6, 1),
                           "frac_mfma": round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4),
                           "traffic": TRAFFIC_BYTES.get(("c3", kname))}
+    # Floors of the access patterns, from the two plain page kernels (one wavefront per 8 KiB row, nothing but
+    # the accesses): the shrink reads x and the weight rows of the adapters in the batch; the expand reads and
+    # writes y (its delta and B^T reads, 5 % of its bytes, are not in the floor).
+    import numpy as np
+    from slora_hip.infer_adapter import page_checksums, page_xor
+    rows = torch.arange(T, dtype=torch.int64, device=device)
+    u = np.unique(seg.ids_np)
+    a_pages = torch.from_numpy(w.a_loc_np[np.concatenate(
+        [w.a_start_np[a] + 3 * w.ranks[a] + np.arange(int(w.ranks[a])) for a in u])]).to(device)
+
+    def read_sweep():
+        for l in range(L):
+            for _ in range(4):
+                page_checksums(x[l], rows)
+                page_checksums(w.key_buffer[l], a_pages)
+
+    def rmw_sweep():
+        for l in range(L):
+            for _ in range(4):
+                page_xor(y[l], rows, 0)
+
+    us_read = time_region(wrap(read_sweep), reps, 3, torch) * 1e3 / (4 * L)
+    us_rmw = time_region(wrap(rmw_sweep), reps, 3, torch) * 1e3 / (4 * L)
+    nb_read = T * H * 2 + int(a_pages.numel()) * w.page_elems * 2
+    kernels["shrink"]["read_only_ceiling"] = {
+        "what": "x rows and one projection's weight rows, loads only (two launches)", "us": round(us_read, 3),
+        "bytes": nb_read, "GBps": round(nb_read / us_read / 1e3, 1),
+        "kernel_over_ceiling": round(kernels["shrink"]["us_per_launch"] / us_read, 3)}
+    kernels["qkv_shrink"]["read_only_ceiling"] = {
+        "what": "the same floor: the fused launch reads x once", "us": round(us_read, 3),
+        "kernel_over_ceiling": round(kernels["qkv_shrink"]["us_per_launch"] / us_read, 3)}
+    kernels["expand"]["rmw_ceiling"] = {
+        "what": "y rows read and written in place, nothing else", "us": round(us_rmw, 3), "bytes": 2 * T * H * 2,
+        "GBps": round(2 * T * H * 2 / us_rmw / 1e3, 1),
+        "kernel_over_ceiling": round(kernels["expand"]["us_per_launch"] / us_rmw, 3)}
+    kernels["qkv_expand"]["rmw_ceiling"] = {
+        "what": "three times the single projection's floor", "us": round(3 * us_rmw, 3),
+        "kernel_over_ceiling": round(kernels["qkv_expand"]["us_per_launch"] / (3 * us_rmw), 3)}
     dom = max((k for n, k in kernels.items() if not n.startswith("qkv_")), key=lambda k: k["us_per_launch"])
     out = {
         "metric": "LoRA prefill tokens/s + achieved HBM GB/s (% peak), C3 segmented shrink/expand",
@@ -728,6 +801,29 @@ def main():
                                                    "GBps": round(nb / us / 1e3, 1),
                                                    "kernel_over_ceiling": round(kernels[label]["us_per_launch"] / us, 3)}
 
+    streaming = None
+    if fused:
+        # what a plain read reaches on this chip when a launch is large: the same checksum kernel over
+        # 16384 neighbouring pages of every layer's pool (as many bytes as a 134 MB launch would move)
+        n_seq = min(16384, w.n_pages)
+        seq = torch.arange(n_seq, dtype=torch.int64, device=device)
+
+        def seq_sweep():
+            for l in range(w.n_layers):
+                page_checksums(w.key_buffer[l], seq)
+
+        fn = graphed(seq_sweep, torch) if use_graph else seq_sweep
+        us = time_region(fn, reps, 3, torch) * 1e3 / w.n_layers
+        nb = n_seq * w.page_elems * 2
+        streaming = {"contiguous_read": {"what": f"{n_seq} neighbouring pages per launch, one wavefront per page, loads only",
+                                         "bytes": nb, "us": round(us, 3), "GBps": round(nb / us / 1e3, 1),
+                                         "frac_of_peak": round(nb / us / 1e3 / HBM_PEAK_GBS, 4)}}
+        # the step if every launch ran at its read-only ceiling
+        ceil_us = sum(k["read_only_ceiling"]["us"] * k["launches_per_step"] for k in kernels.values())
+        streaming["step_at_read_only_ceilings"] = {
+            "ms": round(ceil_us * 1e-3, 4),
+            "frac_of_peak": round(w.step_bytes(fused) / (ceil_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+
     step_gbs = w.step_bytes(fused) / (ms_per_step * 1e-3) / 1e9
     out = {
         "metric": METRIC,
@@ -748,7 +844,7 @@ def main():
             "layers": w.n_layers,
             "batch": w.batch,
             "distinct_adapters_in_batch": int(w.distinct_adapters().size),
-            "pool_pages_per_layer": w.n_pages, "placement": args.placement,
+            "pool_pages_per_layer": w.n_pages, "page_bytes": w.page_elems * 2, "placement": args.placement,
             "mode": args.mode,
             "launch": args.launch,
             "launches_per_step": w.n_layers * (4 if fused else 8) +
@@ -772,8 +868,12 @@ def main():
         },
         "kernels": kernels,
     }
+    if streaming is not None:
+        out["streaming"] = streaming
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, bufs, torch, args.cpu_reps)
+        if args.workload == "s2":
+            out["cpu_baseline"]["c1"] = cpu_baseline_c1(torch)
     if args.workload == "s4" and not args.no_extras:
         # the prefill half of the mixed S4 step, over the same pool: 4 requests of 256 tokens
         pf = measure_prefill(argparse.Namespace(layers=min(w.n_layers, 4), steps=10, warmup=3, launch="graph"), torch,

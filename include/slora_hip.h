@@ -34,7 +34,16 @@
 extern "C" {
 #endif
 
-#define SLORA_VERSION 102 /* 0.1.2: + slora_sgmm_expand_qkv; 0.1.1: + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed, slora_pool_alloc_contiguous_static */
+/* major * 100 + minor.  The major number changes when an entry point is removed or its
+ * signature changes (callers built against an older major must be rebuilt), the minor one when
+ * entry points are added.
+ *   2.0 (200): slora_bgmv_lora_planned (shrink and expand in one launch, present in 1.0 only) is
+ *              gone -- it was removed in 1.1 without a major bump, which this number corrects;
+ *              + slora_pool_page_xor.
+ *   1.2 (102): + slora_sgmm_expand_qkv.
+ *   1.1 (101): + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed,
+ *              slora_pool_alloc_contiguous_static; - slora_bgmv_lora_planned. */
+#define SLORA_VERSION 200
 
 #define SLORA_API __attribute__((visibility("default")))
 
@@ -325,6 +334,14 @@ SLORA_API int slora_pool_gather_a(void* out, int64_t out_cols, const void* pool,
  * reads and reports that as the streaming ceiling of the launch. */
 SLORA_API int slora_pool_page_checksums(uint32_t* out, const void* pool, const int64_t* loc, int64_t n,
                                         int64_t page_bytes, int64_t n_pages, void* stream);
+
+/* In-place xor of pool pages: every 32-bit word of page loc[i] of `pool` ^= key (ids outside
+ * [0, n_pages) are skipped; a page listed twice is undefined).  No counterpart in the reference.
+ * Like slora_pool_page_checksums it is a measurement aid as much as a tool: one wavefront per
+ * page, loads then stores and nothing else, so with key = 0 its duration over the rows of an
+ * output is the read-modify-write floor the benchmark reports next to the expand kernels. */
+SLORA_API int slora_pool_page_xor(void* pool, const int64_t* loc, int64_t n, int64_t page_bytes, int64_t n_pages,
+                                  uint32_t key, void* stream);
 
 /* ---- page allocator over the pool's free map ---------------------------------
  * mem_state: one byte per pool page, 1 = free (the reference's torch.bool

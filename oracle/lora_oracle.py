@@ -18,7 +18,7 @@ the reference checkout):
 * ``ref_prefill_expand``   slora/models/peft/triton_kernel/lora/lora_prefill.py:10-54, 105-136
 * ``ref_var_len_copy``     slora/server/router/model_infer/infer_adapter.py:261-280
 
-Pinning (see tests/test_oracle_*.py): pack/unpack are inverse statements of the
+Pinning (see tests/test_oracle.py): pack/unpack are inverse statements of the
 pool layout taken from two different reference files; the paged restatements
 (index arithmetic over ``a_loc``) must agree with the dense closed form
 ``y + scale * (x @ A) @ B`` evaluated in float64 by numpy, with the reference's

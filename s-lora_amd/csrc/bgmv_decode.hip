@@ -32,8 +32,7 @@ namespace {
 
 constexpr int kTT = 4;                    // most tokens merged into one run
 constexpr int kRB = 8;                    // rows / pages per item
-constexpr int kVecPerPass = 8;            // 16-byte vectors a lane holds per pass over a page
-constexpr int kPassElems = kVecPerPass * kWave * 8;  // 4096 elements
+constexpr int kVecPerPass = 8;            // 16-byte vectors a lane holds per 4096-element pass over a page
 
 struct Tables {
   const int64_t* a_start;
@@ -556,15 +555,27 @@ __device__ __forceinline__ void file_sums(float (&v)[kVecPerPass], float scale, 
 // One page of the flattened (h_out, r) matrix B^T for one run, rank r a power
 // of two (8..128) that divides the page: r/8 lanes share an output, so a
 // wavefront-wide 16-byte load covers 512/r consecutive outputs.  The reduced,
-// scaled sums of a pass are transposed through a 1 KiB LDS strip of the
-// wavefront so that the read-modify-write of y is one 16-byte load and one
-// 16-byte store per lane and token.
+// scaled sums of a pass are transposed through an LDS strip of the wavefront
+// so that the read-modify-write of y is one 16-byte load and one 16-byte store
+// per lane and token.
+// NV: 16-byte vectors a lane holds per pass, i.e. a pass covers 512 * NV elements; the host
+// picks the smallest NV whose pass holds the whole page (8, 10, 12, 16: pages of up to 4096,
+// 5120, 6144, 8192 elements), so that every load of the page is issued before the first wait.
+// Wider pages take several passes.
 // FULL: every element of the page belongs to an output inside h_out and every rank
 // column is used (the caller checks: whole passes, page inside the output, delta as wide
 // as the rank) -- then no load needs its result masked.
-template <typename T, bool FULL>
+template <int NV>
+struct ExpandPass {
+  static constexpr int kElems = NV * kWave * 8;            // elements per pass
+  static constexpr int kGroups = (NV + kVecPerPass - 1) / kVecPerPass;  // groups of 8 loads whose sums are filed together
+  static constexpr int kStrip = kGroups * kVecPerPass * kWave;          // 16-bit entries of a wavefront's LDS strip
+};
+
+template <typename T, bool FULL, int NV>
 __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const Item& it, int r_eff,
                                             const uint16_t* wpage, int64_t flat0, float scale, uint16_t* s_strip) {
+  constexpr int kPass = ExpandPass<NV>::kElems;
   const int lane = threadIdx.x & 63;
   const int r = it.r;
   const int lg_r = __builtin_ctz((unsigned)r);
@@ -572,7 +583,8 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
   const int d0 = (lane & (lpo - 1)) * 8;
   const bool d_ok = FULL || d0 < r_eff;
   const int page_elems = (int)p.page_elems;
-  const int out_per_pass = kPassElems >> lg_r;
+  const int out_per_pass = kPass >> lg_r;
+  const int opw = kWave >> (lg_r - 3);  // outputs a wavefront-wide load covers
   const int n_page0 = (int)(flat0 >> lg_r);  // first output of this page
   // outputs of this page: [n_page0, n_end); later pages own what lies beyond
   const int n_page_end = n_page0 + (page_elems >> lg_r);
@@ -582,9 +594,9 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
   const uint16_t* x = reinterpret_cast<const uint16_t*>(p.x[proj]);
 
   // first pass of the page and the run's delta fragments go in flight together
-  u32x4 wv[kVecPerPass];
+  u32x4 wv[NV];
 #pragma unroll
-  for (int c = 0; c < kVecPerPass; ++c) {
+  for (int c = 0; c < NV; ++c) {
     const int e = (c * kWave + lane) * 8;
     if (FULL) {
       wv[c] = ldg16_stream(wpage + e);
@@ -602,10 +614,10 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
       xv[t] = (t < it.n_tok && d_ok) ? ldg16(x + (int64_t)it.tok[t] * p.x_cols + d0) : zero16();
   }
 
-  for (int e0 = 0; e0 < page_elems; e0 += kPassElems) {
+  for (int e0 = 0; e0 < page_elems; e0 += kPass) {
     if (e0 != 0) {
 #pragma unroll
-      for (int c = 0; c < kVecPerPass; ++c) {
+      for (int c = 0; c < NV; ++c) {
         const int e = e0 + (c * kWave + lane) * 8;
         if (FULL) {
           wv[c] = ldg16_stream(wpage + e);
@@ -615,8 +627,10 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
         }
       }
     }
-    // this lane's 8 consecutive outputs of the pass
-    const int n_mine = n_page0 + (e0 >> lg_r) + lane * 8;
+    // this lane's 8 consecutive outputs of the pass (of its first 512 outputs: a pass has more
+    // only for rank 8 and NV > 8, and those follow in further steps)
+    const int n_pass0 = n_page0 + (e0 >> lg_r);
+    const int n_mine = n_pass0 + lane * 8;
     const bool y_ok = lane * 8 < out_per_pass && n_mine < n_end;
     u32x4 yv[kTT];
 #pragma unroll
@@ -632,15 +646,22 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
     for (int t = 0; t < kTT; ++t) {
       if (t < it.n_tok) {
-        float part[kVecPerPass];
+        // partial sums of the pass, eight loads at a time (a last group of fewer loads is
+        // padded with zeros, which add nothing)
 #pragma unroll
-        for (int c = 0; c < kVecPerPass; ++c) part[c] = dot8<T>(wv[c], xv[t], 0.f);
-        switch (lpo) {
-          case 1: file_sums<T, 1>(part, scale, lane, s_strip); break;
-          case 2: file_sums<T, 2>(part, scale, lane, s_strip); break;
-          case 4: file_sums<T, 4>(part, scale, lane, s_strip); break;
-          case 8: file_sums<T, 8>(part, scale, lane, s_strip); break;
-          default: file_sums<T, 16>(part, scale, lane, s_strip); break;
+        for (int g8 = 0; g8 < ExpandPass<NV>::kGroups; ++g8) {
+          float part[kVecPerPass];
+#pragma unroll
+          for (int c = 0; c < kVecPerPass; ++c)
+            part[c] = g8 * kVecPerPass + c < NV ? dot8<T>(wv[g8 * kVecPerPass + c], xv[t], 0.f) : 0.f;
+          uint16_t* strip = s_strip + g8 * kVecPerPass * opw;
+          switch (lpo) {
+            case 1: file_sums<T, 1>(part, scale, lane, strip); break;
+            case 2: file_sums<T, 2>(part, scale, lane, strip); break;
+            case 4: file_sums<T, 4>(part, scale, lane, strip); break;
+            case 8: file_sums<T, 8>(part, scale, lane, strip); break;
+            default: file_sums<T, 16>(part, scale, lane, strip); break;
+          }
         }
         // the same wavefront wrote the strip: its LDS operations complete in order
         const u32x4 dv = *reinterpret_cast<const u32x4*>(s_strip + (y_ok ? lane * 8 : 0));
@@ -649,6 +670,21 @@ __device__ __forceinline__ void expand_page(const ExpandArgs& p, int proj, const
 #pragma unroll
           for (int q = 0; q < 4; ++q) out[q] = T::add2(yv[t][q], dv[q]);
           stg16_stream(y + (int64_t)it.tok[t] * h_stride + n_mine, out);
+        }
+        if (NV > kVecPerPass) {
+          // outputs 512.. of the pass (rank 8 only): y is loaded here, behind the sums
+          for (int s0 = 8 * kWave; s0 < out_per_pass; s0 += 8 * kWave) {
+            const int n2 = n_pass0 + s0 + lane * 8;
+            if (s0 + lane * 8 < out_per_pass && n2 < n_end) {
+              uint16_t* yp = y + (int64_t)it.tok[t] * h_stride + n2;
+              const u32x4 y2 = ldg16_stream(yp);
+              const u32x4 d2 = *reinterpret_cast<const u32x4*>(s_strip + s0 + lane * 8);
+              u32x4 out;
+#pragma unroll
+              for (int q = 0; q < 4; ++q) out[q] = T::add2(y2[q], d2[q]);
+              stg16_stream(yp, out);
+            }
+          }
         }
       }
     }
@@ -690,7 +726,7 @@ __device__ __forceinline__ void expand_scalar(const ExpandArgs& p, int proj, con
 
 // Page kk of projection `proj` for the item's run; `page` is its pool page id
 // or -2 to look it up in a_loc.
-template <typename T>
+template <typename T, int NV>
 __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const Item& it, int r_eff, int kk,
                                            int64_t page, bool vec_ok, uint16_t* s_strip) {
   const int64_t base_li = it.base + (int64_t)it.r * (p.qkvo0 + proj);
@@ -704,12 +740,12 @@ __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const 
   const int64_t flat0 = (int64_t)kk * p.page_elems;
   const float scale = load_scale(p.scales, p.scales_dtype, it.a);
   // the whole page lies inside the output, in whole passes, and delta is as wide as the rank
-  const bool full = r_eff == it.r && (p.page_elems & (kPassElems - 1)) == 0 &&
+  const bool full = r_eff == it.r && p.page_elems % ExpandPass<NV>::kElems == 0 &&
                     flat0 + p.page_elems <= (int64_t)p.h_out[proj] * it.r;
   if (full)
-    expand_page<T, true>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
+    expand_page<T, true, NV>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
   else
-    expand_page<T, false>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
+    expand_page<T, false, NV>(p, proj, it, r_eff, wpage, flat0, scale, s_strip);
 }
 
 // Expand has nothing to share between wavefronts (the delta row is 16 bytes per
@@ -719,7 +755,7 @@ __device__ __forceinline__ void expand_one(const ExpandArgs& p, int proj, const 
 // Grid: x = item (planned) or token * blocks + block (stateless), y = projection * 2 +
 // half: workgroup ids run item-fastest, so with a multiple of 8 items every workgroup of
 // an item lands on XCD item % 8.
-template <typename T, int NPROJ, bool PLANNED>
+template <typename T, int NPROJ, bool PLANNED, int NV>
 __device__ __forceinline__ int expand_body(const ExpandArgs& p, int unit, int sub, uint16_t* s_strip) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int proj = sub >> 1;
@@ -765,11 +801,11 @@ __device__ __forceinline__ int expand_body(const ExpandArgs& p, int unit, int su
                       (p.page_elems & (8 * r - 1)) == 0 && (p.h_out[proj] & 7) == 0 && p.y_aligned != 0;
   if (k < n_pg) {
     const int64_t page = PLANNED ? (int64_t)plan_pg : (int64_t)-2;
-    expand_one<T>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
+    expand_one<T, NV>(p, proj, it, r_eff, k, page, vec_ok, s_strip);
   }
   if (extra) {
 #pragma unroll 1
-    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
+    for (int kk = k + kRB; kk < n_pg; kk += kRB) expand_one<T, NV>(p, proj, it, r_eff, kk, -2, vec_ok, s_strip);
   }
   return it.plan_items;
 }
@@ -1407,9 +1443,6 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
 // Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
 // more of them resident hide more of each other's waits), four for a single projection (all of
 // its workgroups are resident at once, and four leave 128 registers: nothing spills).
-// Five workgroups per compute unit for the q/k/v launch (its 3000 workgroups come in rounds,
-// more of them resident hide more of each other's waits), four for a single projection (all of
-// its workgroups are resident at once, and four leave 128 registers: nothing spills).
 // Grid, two forms.  Two-dimensional (x = unit, y = projection * 2 + half): all workgroups of
 // one projection half run before those of the next.  One-dimensional (p.interleave): id L
 // -> unit 8 * (L / (8 * S)) + L % 8, sub (L / 8) % S with S = 2 * NPROJ, so a unit still sits
@@ -1417,9 +1450,12 @@ int launch_shrink(ShrinkArgs p, int nproj, int64_t units, hipStream_t stream) {
 // narrower than a page (grouped-query k and v): most of their workgroups find no page and
 // exit, and spread between the others they cost nothing, while in phases of their own they
 // are all a phase consists of.
-template <typename T, int NPROJ, bool PLANNED>
-__global__ __launch_bounds__(256, NPROJ == 3 ? 5 : 4) void bgmv_expand_kernel(const ExpandArgs p) {
-  __shared__ __align__(16) uint16_t s_out[4][kPassElems / 8];
+// NV: see expand_page.  The wider instantiations hold more of a page in registers and get one
+// workgroup per compute unit fewer.
+template <typename T, int NPROJ, bool PLANNED, int NV>
+__global__ __launch_bounds__(256, NV > 8 ? (NV > 12 ? 3 : 4) : (NPROJ == 3 ? 5 : 4)) void bgmv_expand_kernel(
+    const ExpandArgs p) {
+  __shared__ __align__(16) uint16_t s_out[4][ExpandPass<NV>::kStrip];
   int unit = (int)blockIdx.x, sub = (int)blockIdx.y;
   if (p.interleave) {
     constexpr int S = 2 * NPROJ;
@@ -1428,12 +1464,20 @@ __global__ __launch_bounds__(256, NPROJ == 3 ? 5 : 4) void bgmv_expand_kernel(co
     sub = g % S;
     if (unit >= p.n_units) return;
   }
-  const int n_items = expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
+  const int n_items = expand_body<T, NPROJ, PLANNED, NV>(p, unit, sub, s_out[threadIdx.x >> 6]);
   if (PLANNED && p.strided) {  // the items beyond the grid, if the batch has that many
     const int stride = p.interleave ? (int)gridDim.x / (2 * NPROJ) : (int)gridDim.x;  // units of the grid
     for (unit += stride; unit < n_items; unit += stride)
-      expand_body<T, NPROJ, PLANNED>(p, unit, sub, s_out[threadIdx.x >> 6]);
+      expand_body<T, NPROJ, PLANNED, NV>(p, unit, sub, s_out[threadIdx.x >> 6]);
   }
+}
+
+template <typename T, int NPROJ, bool PLANNED, int NV>
+int launch_expand_nv(ExpandArgs p, int64_t items, hipStream_t stream) {
+  dim3 grid((uint32_t)items, 2 * NPROJ);
+  if (p.interleave) grid = dim3((uint32_t)((items + 7) / 8 * 8 * 2 * NPROJ), 1);
+  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED, NV>), grid, dim3(256), 0, stream, p);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 
 template <typename T, int NPROJ, bool PLANNED>
@@ -1444,10 +1488,15 @@ int launch_expand(ExpandArgs p, int64_t items, hipStream_t stream) {
   p.interleave = 0;
   for (int i = 0; i < NPROJ; ++i)
     if (p.pages_shift[i] > 0) p.interleave = 1;  // an output narrower than a page
-  dim3 grid((uint32_t)items, 2 * NPROJ);
-  if (p.interleave) grid = dim3((uint32_t)((items + 7) / 8 * 8 * 2 * NPROJ), 1);
-  hipLaunchKernelGGL((bgmv_expand_kernel<T, NPROJ, PLANNED>), grid, dim3(256), 0, stream, p);
-  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+  // planned launches: the instantiation whose pass holds the whole page (the stateless kernels keep
+  // the 4096-element pass)
+  if (PLANNED) {
+    const int64_t pv = p.page_elems >> 3;
+    if (pv > 8 * kWave && pv <= 10 * kWave) return launch_expand_nv<T, NPROJ, PLANNED, PLANNED ? 10 : 8>(p, items, stream);
+    if (pv > 10 * kWave && pv <= 12 * kWave) return launch_expand_nv<T, NPROJ, PLANNED, PLANNED ? 12 : 8>(p, items, stream);
+    if (pv > 12 * kWave && pv <= 16 * kWave) return launch_expand_nv<T, NPROJ, PLANNED, PLANNED ? 16 : 8>(p, items, stream);
+  }
+  return launch_expand_nv<T, NPROJ, PLANNED, 8>(p, items, stream);
 }
 
 template <typename T>
@@ -1685,16 +1734,9 @@ int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* ta
     int n = 64;
     while (n < batch) n <<= 1;
     const size_t lds = (size_t)n * 4 + (size_t)(n + 1) * 4 + (size_t)n * 2 + 16;
-    static bool attr_done = false;  // benign if two threads race: the call is idempotent
-    if (!attr_done) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(bgmv_plan_sort_kernel),
-                              hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kSortPlanBatch * 10 + 32) != hipSuccess) {
-        (void)hipGetLastError();
-        return SLORA_ERR_LAUNCH;
-      }
-      attr_done = true;
-    }
+    static PerDeviceOnce once;
+    if (!raise_dynamic_lds(reinterpret_cast<const void*>(bgmv_plan_sort_kernel), kSortPlanBatch * 10 + 32, once))
+      return SLORA_ERR_LAUNCH;
     int64_t grid = (max_items + kPlanThreads / 16 - 1) / (kPlanThreads / 16);
     grid = grid < 1 ? 1 : (grid > 16 ? 16 : grid);
     hipLaunchKernelGGL(bgmv_plan_sort_kernel, dim3((uint32_t)grid), dim3(kPlanThreads), lds,

@@ -360,6 +360,34 @@ __global__ __launch_bounds__(256) void page_xor_kernel(const u32x4* __restrict__
   if (lane == 0) out[i] = r;
 }
 
+// The same walk with a write: every 32-bit word of page loc[i] is xor-ed with `key` in place
+// (key 0 leaves the data as it is and still reads and writes every byte).  One wavefront per
+// page, all loads of a pass issued before the first store: the plainest read-modify-write of
+// scattered rows, timed by the benchmark as the floor of the kernels that update an output in
+// place (the expand kernels' y).
+__global__ __launch_bounds__(256) void page_rmw_kernel(u32x4* __restrict__ pool, int64_t page_vecs, int64_t n_pages,
+                                                       const int64_t* __restrict__ loc, int64_t n, uint32_t key) {
+  const int lane = threadIdx.x & 63;
+  const int64_t i = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int64_t page = loc[i];
+  if ((uint64_t)page >= (uint64_t)n_pages) return;
+  u32x4* row = pool + page * page_vecs;
+  for (int64_t v0 = 0; v0 < page_vecs; v0 += 8 * kWave) {
+    u32x4 v[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int64_t k = v0 + c * kWave + lane;
+      v[c] = k < page_vecs ? ldg16_stream(row + k) : zero16();
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      const int64_t k = v0 + c * kWave + lane;
+      if (k < page_vecs) stg16_stream(row + k, v[c] ^ u32x4{key, key, key, key});
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // page allocator over the free map (1 byte per page, 1 = free)
 // ---------------------------------------------------------------------------
@@ -749,6 +777,21 @@ int slora_pool_page_checksums(uint32_t* out, const void* pool, const int64_t* lo
   if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(page_xor_kernel, dim3((uint32_t)grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
                      static_cast<const u32x4*>(pool), page_bytes / 16, n_pages, loc, n, out);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
+int slora_pool_page_xor(void* pool, const int64_t* loc, int64_t n, int64_t page_bytes, int64_t n_pages, uint32_t key,
+                        void* stream) {
+  using namespace slora;
+  if (n < 0 || page_bytes < 0 || n_pages < 0) return SLORA_ERR_BAD_SHAPE;
+  if (n == 0) return SLORA_OK;
+  if (pool == nullptr || loc == nullptr) return SLORA_ERR_NULL_POINTER;
+  if (page_bytes % 16 != 0) return SLORA_ERR_UNSUPPORTED;
+  if (!aligned16(pool)) return SLORA_ERR_ALIGNMENT;
+  const int64_t grid = (n + 3) / 4;
+  if (grid > 0x7fffffffLL) return SLORA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(page_rmw_kernel, dim3((uint32_t)grid), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     static_cast<u32x4*>(pool), page_bytes / 16, n_pages, loc, n, key);
   return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
 }
 

@@ -1406,14 +1406,8 @@ int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t strea
   if (plan != nullptr && !shrink_plan_usable(p.t.n_requests, p.m_tiles, grid, q.col_split)) return SLORA_ERR_BAD_SHAPE;
   const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ, DEEP>)
                                        : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ, DEEP>);
-  static bool attr_done[2] = {false, false};  // benign if two threads race: the call is idempotent
-  if (!attr_done[plan != nullptr]) {
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) {
-      (void)hipGetLastError();
-      return SLORA_ERR_LAUNCH;
-    }
-    attr_done[plan != nullptr] = true;
-  }
+  static PerDeviceOnce once[2];
+  if (!raise_dynamic_lds(kernel, (int)lds, once[plan != nullptr])) return SLORA_ERR_LAUNCH;
   if (plan != nullptr)
     hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ, DEEP>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q,
                        plan);
@@ -1427,15 +1421,9 @@ int launch_seg_expand_ks(const SegExpandArgs& p, int64_t grid, hipStream_t strea
   const bool walk = p.t.n_requests <= kExpReqs && p.t.n_tokens <= (1 << 22);  // tile counts stay far inside 32 bits
   auto kernel = walk ? sgmm_expand_walk_kernel<T, KS, NPROJ> : sgmm_expand_kernel<T, KS, NPROJ>;
   constexpr int lds = 2 * kExpChunkRows * kExpLdsRow<KS>;  // 68 KiB for ranks up to 128
-  static bool attr_done[2] = {lds <= 64 * 1024, lds <= 64 * 1024};  // benign if two threads race: the call is idempotent
-  if (!attr_done[walk]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            lds) != hipSuccess) {
-      (void)hipGetLastError();
-      return SLORA_ERR_LAUNCH;
-    }
-    attr_done[walk] = true;
-  }
+  static PerDeviceOnce once[2];
+  if (lds > 64 * 1024 && !raise_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, once[walk]))
+    return SLORA_ERR_LAUNCH;
   if (walk) {
     // as many slices per output group as fill the chip, at most one per row tile
     const int64_t tiles = ((int64_t)p.t.n_tokens + kExpTMW - 1) / kExpTMW + p.t.n_requests;

@@ -963,6 +963,21 @@ Tensor page_checksums(const Tensor& buffer, const Tensor& loc) {
   return out;
 }
 
+// buffer[loc[i]] ^= key on every 32-bit word, in place (key 0: a pure read-modify-write)
+void page_xor(Tensor& buffer, const Tensor& loc, int64_t key) {
+  SL_CHECK_INPUT(buffer);
+  SL_CHECK_INPUT(loc);
+  SL_CHECK_INDEX(loc);
+  TORCH_CHECK(buffer.dim() >= 1, "buffer must be [pages, ...]");
+  TORCH_CHECK(key >= 0 && key <= 0xffffffffLL, "key must fit 32 bits");
+  const int64_t n_pages = buffer.size(0);
+  const int64_t page_bytes = n_pages > 0 ? buffer.numel() / n_pages * buffer.element_size() : 0;
+  const int rc = slora_pool_page_xor(buffer.data_ptr(), loc.data_ptr<int64_t>(), loc.numel(), page_bytes, n_pages,
+                                     static_cast<uint32_t>(key), stream_of(buffer));
+  check_rc(rc, "page_xor");
+  mark_written(buffer);
+}
+
 Tensor gather_lora_a(const Tensor& key_buffer, const Tensor& a_loc, int64_t first, int64_t rank, int64_t hidden,
                      int64_t out_cols) {
   SL_CHECK_INPUT(key_buffer);
@@ -1060,6 +1075,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         py::arg("result"), py::arg("work") = py::none());
   m.def("pool_free", &pool_free);
   m.def("page_checksums", &page_checksums, py::arg("buffer"), py::arg("loc"));
+  m.def("page_xor", &page_xor, py::arg("buffer"), py::arg("loc"), py::arg("key") = 0);
   m.def("gather_lora_a", &gather_lora_a, py::arg("key_buffer"), py::arg("a_loc"), py::arg("first"), py::arg("rank"),
         py::arg("hidden"), py::arg("out_cols") = 0);
 }

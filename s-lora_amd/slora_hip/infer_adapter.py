@@ -101,6 +101,13 @@ def page_checksums(buffer: torch.Tensor, loc: torch.Tensor) -> torch.Tensor:
     return _kernels.page_checksums(buffer, loc)
 
 
+def page_xor(buffer: torch.Tensor, loc: torch.Tensor, key: int = 0) -> None:
+    """``buffer[loc[i]] ^= key`` on every 32-bit word, in place.  With ``key = 0`` nothing changes
+    but every listed page is read and written once: the plain read-modify-write of scattered
+    rows that the benchmark times as the floor of the kernels that update an output in place."""
+    _kernels.page_xor(buffer, loc, int(key))
+
+
 def gather_lora_a(key_buffer, a_loc, first: int, rank: int, hidden: int, out_cols: int = 0) -> torch.Tensor:
     """``A_p`` as a dense ``[hidden, out_cols]`` tensor out of the pool pages
     ``a_loc[first : first + rank]`` (lora_single_batch_infer.py:38-46); columns

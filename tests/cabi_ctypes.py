@@ -68,6 +68,7 @@ SIGNATURES = {
     "slora_pool_alloc_contiguous_static": (_I, [_P, _I64, _I64, _P, _P, _P]),
     "slora_pool_free": (_I, [_P, _I64, _P, _I64, _P]),
     "slora_pool_page_checksums": (_I, [_P, _P, _P, _I64, _I64, _I64, _P]),
+    "slora_pool_page_xor": (_I, [_P, _P, _I64, _I64, _I64, C.c_uint32, _P]),
 }
 
 _lib = None

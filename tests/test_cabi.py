@@ -39,7 +39,7 @@ def test_header_and_binding_agree(lib):
 
 def test_version_and_strerror(lib):
     import cabi_ctypes as _cabi
-    assert lib.slora_version() == 102
+    assert lib.slora_version() == 200
     assert _cabi.strerror(0) == "ok"
     assert "No suitable kernel" in _cabi.strerror(_cabi.ERR_UNSUPPORTED)
     for code in range(-7, 0):

@@ -481,3 +481,21 @@ def test_page_checksums_equal_numpy_xor(gpu, dtype, heads, head_dim):
     assert np.array_equal(got[ok], want[loc[ok]])
     assert np.all(got[~ok] == 0)
     assert page_checksums(buf, torch.empty(0, dtype=torch.int64, device=gpu)).numel() == 0
+
+
+def test_page_xor_is_an_exact_in_place_xor(gpu):
+    """page_xor against numpy: listed pages ^= key word by word, other pages and ids outside the
+    buffer untouched, key 0 and an empty list change nothing."""
+    from slora_hip.infer_adapter import page_xor
+    rng = np.random.default_rng(13)
+    words = rng.integers(0, 2 ** 32, size=(200, 640), dtype=np.uint64).astype(np.uint32)   # 2560-byte pages
+    buf = torch.from_numpy(words.view(np.int32)).to(gpu)
+    loc = rng.permutation(200)[:77].astype(np.int64)
+    loc_dev = torch.from_numpy(np.concatenate([loc, [-1, 200]])).to(gpu)
+    page_xor(buf, loc_dev, 0)
+    page_xor(buf, torch.empty(0, dtype=torch.int64, device=gpu), 0x5a5a5a5a)
+    assert np.array_equal(buf.cpu().numpy().view(np.uint32), words)
+    page_xor(buf, loc_dev, 0x9e3779b9)
+    want = words.copy()
+    want[loc] ^= np.uint32(0x9e3779b9)
+    assert np.array_equal(buf.cpu().numpy().view(np.uint32), want)
