@@ -51,11 +51,12 @@ def parse_args():
                     help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels; "
                          "load: copying adapters into the pool; the last two are reported in the same format with "
                          "their own metric names")
-    ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused"],
+    ap.add_argument("--mode", choices=["dropin", "fused", "planned", "planned-fused", "planned-lora"],
                     default="planned-fused",
                     help="dropin: 8 stateless dispatch_bgmv calls per layer exactly as the reference issues them; "
                          "fused: q/k/v shrink and q/k/v expand as one launch each (4 launches per layer); "
-                         "planned*: the same with a per-step plan (built inside every timed step) passed as plan=")
+                         "planned*: the same with a per-step plan (built inside every timed step) passed as plan=; "
+                         "planned-lora: shrink and expand of q/k/v in one launch and of o in one launch (2 per layer)")
     ap.add_argument("--all-modes", action="store_true", help="also time the other modes and report them under 'modes'")
     ap.add_argument("--launch", choices=["graph", "direct"], default="graph",
                     help="graph: the step is captured once into a HIP graph and replayed; direct: Python calls")
@@ -108,7 +109,8 @@ def make_step(w, bufs, mode, keep_plan=False):
     bgmv = slora_hip.dispatch_bgmv
     t = (w.a_start, w.a_len, w.a_loc, w.req_bins)
     planned = mode.startswith("planned")
-    fused = mode.endswith("fused")
+    one_launch = mode == "planned-lora"
+    fused = mode.endswith("fused") or one_launch
     plan = slora_hip.make_plan(*t, w.max_rank, w.n_pages) if planned else None
     kw = {"plan": plan} if planned else {}
     L = w.n_layers
@@ -129,6 +131,15 @@ def make_step(w, bufs, mode, keep_plan=False):
     def expand(l, p):
         bgmv(bufs.y[l][p], bufs.delta[p % 3], w.value_buffer[l], *t, p, w.a_scaling, **kw)
 
+    def qkv_lora(l):
+        slora_hip.dispatch_bgmv_qkv_lora(bufs.y[l][0], bufs.y[l][1], bufs.y[l][2], bufs.delta[0], bufs.delta[1],
+                                         bufs.delta[2], bufs.x_in[l], w.key_buffer[l], w.value_buffer[l], *t,
+                                         w.a_scaling, **kw)
+
+    def o_lora(l):
+        slora_hip.dispatch_bgmv_lora(bufs.y[l][3], bufs.delta[0], bufs.x_att[l], w.key_buffer[l], w.value_buffer[l], *t,
+                                     3, w.a_scaling, **kw)
+
     def over_layers(fn, *a):
         def sweep():
             for l in range(L):
@@ -144,7 +155,13 @@ def make_step(w, bufs, mode, keep_plan=False):
 
     nv = next((n for n in (8, 10, 12, 16) if w.hidden <= 512 * n), 8)  # the instantiation the library picks
     sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}, {nv}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
-    if fused:
+    if one_launch:
+        lk = f"bgmv_lora_kernel<{ty}, %d, {nv}>"
+        families = {
+            "qkv_lora": (over_layers(qkv_lora), lk % 3, L, w.qkv_shrink_bytes() + w.qkv_expand_bytes()),
+            "o_lora": (over_layers(o_lora), lk % 1, L, w.shrink_bytes() + w.expand_bytes(w.h_out[3])),
+        }
+    elif fused:
         families = {
             "qkv_shrink": (over_layers(qkv_shrink), sk, L, w.qkv_shrink_bytes()),
             "o_shrink": (over_layers(shrink, 3), sk, L, w.shrink_bytes()),
@@ -164,6 +181,10 @@ def make_step(w, bufs, mode, keep_plan=False):
             # a new batch every step: calls that pass no plan may reuse one only within the step
             slora_hip.clear_plan_cache()
         for l in range(L):
+            if one_launch:
+                qkv_lora(l)
+                o_lora(l)
+                continue
             if fused:
                 qkv_shrink(l)
                 qkv_expand(l)
@@ -710,7 +731,7 @@ def main():
                                 placement=args.placement)
     bufs = StepBuffers(w, device)
     step, families = make_step(w, bufs, args.mode, args.keep_plan)
-    fused = args.mode.endswith("fused")
+    fused = args.mode.endswith("fused") or args.mode == "planned-lora"
     if args.check:
         check_layer0(w, bufs, torch)
 
@@ -750,14 +771,14 @@ def main():
     spread = step_percentiles(run_step) if use_graph else None
     other_modes = {}
     if args.all_modes:
-        for m in ("dropin", "fused", "planned", "planned-fused"):
+        for m in ("dropin", "fused", "planned", "planned-fused", "planned-lora"):
             if m == args.mode:
                 continue
             st, _ = make_step(w, bufs, m)
             fn = graphed(st, torch) if use_graph else st
             ms = time_steps(fn)
             other_modes[m] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(w.batch / (ms * 1e-3), 1),
-                              "launches_per_step": w.n_layers * (4 if m.endswith("fused") else 8)}
+                              "launches_per_step": w.n_layers * (2 if m == "planned-lora" else 4 if m.endswith("fused") else 8)}
 
     # ---- launch duration of every kind of launch in the step: a sweep of that kind over
     # all layers, HIP events on the stream the kernels run on (back-to-back launches, so
@@ -786,18 +807,24 @@ def main():
             idx = [w.a_start_np[a] + p * w.ranks[a] + np.arange(n_pages(a, p)) for p in projs for a in u]
             return torch.from_numpy(w.a_loc_np[np.concatenate(idx)]).to(device)
 
-        for label, projs, side in (("qkv_shrink", (0, 1, 2), w.key_buffer), ("o_shrink", (3,), w.key_buffer),
-                                   ("qkv_expand", (0, 1, 2), w.value_buffer), ("o_expand", (3,), w.value_buffer)):
-            loc = pages_of(projs, label.endswith("expand"))
+        one_launch = args.mode == "planned-lora"
+        kinds = ((("qkv_lora", (0, 1, 2)), ("o_lora", (3,))) if one_launch else
+                 (("qkv_shrink", (0, 1, 2)), ("o_shrink", (3,)), ("qkv_expand", (0, 1, 2)), ("o_expand", (3,))))
+        for label, projs in kinds:
+            # a launch that does both halves reads the A pages and then the B pages: two checksum launches
+            sides = ([(w.key_buffer, False), (w.value_buffer, True)] if one_launch else
+                     [(w.value_buffer, True)] if label.endswith("expand") else [(w.key_buffer, False)])
+            locs = [(side, pages_of(projs, expand)) for side, expand in sides]
 
-            def sweep(loc=loc, side=side):
+            def sweep(locs=locs):
                 for l in range(w.n_layers):
-                    page_checksums(side[l], loc)
+                    for side, loc in locs:
+                        page_checksums(side[l], loc)
 
             fn = graphed(sweep, torch) if use_graph else sweep
             us = time_region(fn, reps, 3, torch) * 1e3 / w.n_layers
-            nb = int(loc.numel()) * w.page_elems * 2
-            kernels[label]["read_only_ceiling"] = {"us": round(us, 3), "page_bytes": nb,
+            nb = sum(int(loc.numel()) for _, loc in locs) * w.page_elems * 2
+            kernels[label]["read_only_ceiling"] = {"us": round(us, 3), "page_bytes": nb, "launches": len(locs),
                                                    "GBps": round(nb / us / 1e3, 1),
                                                    "kernel_over_ceiling": round(kernels[label]["us_per_launch"] / us, 3)}
 
@@ -847,7 +874,7 @@ def main():
             "pool_pages_per_layer": w.n_pages, "page_bytes": w.page_elems * 2, "placement": args.placement,
             "mode": args.mode,
             "launch": args.launch,
-            "launches_per_step": w.n_layers * (4 if fused else 8) +
+            "launches_per_step": w.n_layers * (2 if args.mode == "planned-lora" else 4 if fused else 8) +
                                  (1 if args.mode.startswith("planned") else 0),
         },
         "step_hbm": {

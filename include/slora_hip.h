@@ -37,9 +37,10 @@ extern "C" {
 /* major * 100 + minor.  The major number changes when an entry point is removed or its
  * signature changes (callers built against an older major must be rebuilt), the minor one when
  * entry points are added.
- *   2.0 (200): slora_bgmv_lora_planned (shrink and expand in one launch, present in 1.0 only) is
- *              gone -- it was removed in 1.1 without a major bump, which this number corrects;
- *              + slora_pool_page_xor.
+ *   2.0 (200): slora_bgmv_lora_planned (shrink and expand in one launch) has a new signature and a
+ *              new plan layout behind it -- the 1.0 form was removed in 1.1 without a major bump,
+ *              which this number corrects; plans hold hand-over counters (slora_bgmv_plan_bytes
+ *              grew); + slora_pool_page_xor.
  *   1.2 (102): + slora_sgmm_expand_qkv.
  *   1.1 (101): + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed,
  *              slora_pool_alloc_contiguous_static; - slora_bgmv_lora_planned. */
@@ -167,6 +168,29 @@ SLORA_API int slora_bgmv_expand_planned(const void* plan, int64_t rank_cap, int6
                                         int64_t batch, int64_t x_cols, int64_t h_out0,
                                         int64_t h_out1, int64_t h_out2, int64_t page_elems,
                                         int64_t n_pages, int qkvo, int dtype, void* stream);
+
+/* Shrink and expand of a projection (nproj = 1) or of q, k and v (nproj = 3, qkvo = 0) in ONE
+ * launch, with a plan.  The reference issues the two back to back for every projection
+ * (slora/models/peft/lora_unordered_batch_infer.py:267-273, 287-293, 307-313, 438-444); here one
+ * workgroup per plan item computes its 8 rows of delta = x A, hands them to the other
+ * workgroups of its run through counters behind the plan (device-scope stores and loads, no
+ * second launch), and then updates y with its 8 pages of B^T:
+ *   delta_i[b, j] = T(sum_k w_a[page(a,p,j), k] * x[b, k])                    as slora_bgmv_shrink
+ *   y_i[b, n]     = T(y_i[b, n] + T(scales[a] * sum_d Bt[n*r+d] * delta_i[b, d]))  as slora_bgmv_expand
+ * bit for bit what the two calls give.  delta_i ([batch, delta_cols], delta_cols a multiple of 8
+ * and at least every rank in the batch for the usual result) is left filled as after the
+ * shrink call.  w_a / w_b are the pools of the A side and the B side (key_buffer[l],
+ * value_buffer[l]), which share page ids.  `plan` is written to (its counters): launches that
+ * use one plan must not overlap, e.g. stay on one stream.  A hand-over that is not complete
+ * after 65536 polls is abandoned (the workgroup goes on and a flag is set behind the plan)
+ * rather than waited for for ever; it never is unless workgroups are not handed out in order. */
+SLORA_API int slora_bgmv_lora_planned(void* plan, int64_t rank_cap, int64_t n_items, int nproj, void* y0, void* y1,
+                                      void* y2, void* delta0, void* delta1, void* delta2, const void* x,
+                                      const void* w_a, const void* w_b, const slora_tables* tables,
+                                      const int64_t* bins, const void* scales, int scales_dtype, int64_t batch,
+                                      int64_t h_in, int64_t delta_cols, int64_t h_out0, int64_t h_out1,
+                                      int64_t h_out2, int64_t page_elems, int64_t n_pages, int qkvo, int dtype,
+                                      void* stream);
 
 /* Prefill (segmented) shrink.  Replaces lora_get_qkvo_fwd_shrink + _shrink_fwd_kernel
  * (slora/models/peft/triton_kernel/lora/lora_prefill.py:139-164, 57-102).

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libslora_hip.so")
 
-SOURCES = ["cabi.hip", "bgmv_decode.hip", "sgmm_prefill.hip", "pool_ops.hip"]
+SOURCES = ["cabi.hip", "bgmv_decode.hip", "bgmv_lora.hip", "sgmm_prefill.hip", "pool_ops.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

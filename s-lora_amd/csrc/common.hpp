@@ -85,6 +85,23 @@ __device__ __forceinline__ void stg16_stream(void* p, u32x4 v) {
 }
 __device__ __forceinline__ u32x4 zero16() { return u32x4{0u, 0u, 0u, 0u}; }
 
+// Values one workgroup writes and another workgroup of the SAME launch reads (the shrink
+// results that the expand half of a one-launch LoRA consumes): relaxed atomics at device
+// scope, which go through to the level every XCD sees instead of a line that one XCD's L2
+// or a compute unit's vector cache may still hold.  Between launches plain accesses do.
+__device__ __forceinline__ u32x4 ldg16_coherent(const void* p) {
+  const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
+  const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint64_t b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return u32x4{(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+}
+__device__ __forceinline__ uint16_t ld16_coherent(const uint16_t* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st16_coherent(uint16_t* p, uint16_t v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // acc += sum_i f32(w_i) * f32(x_i) over the 8 elements of two 16-byte vectors
 template <typename T>
 __device__ __forceinline__ float dot8(u32x4 w, u32x4 x, float acc) {

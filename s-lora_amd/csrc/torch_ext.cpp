@@ -494,6 +494,103 @@ void dispatch_bgmv_qkv_expand(const Tensor& y_q, const Tensor& y_k, const Tensor
   check_rc(rc, "dispatch_bgmv_qkv_expand");
 }
 
+// Shrink and expand of one projection in one launch: delta = x A (left in `delta`), y += scale * delta B.
+// With plan=False (or no plan for the batch) the two stateless launches are issued instead.
+void dispatch_bgmv_lora(const Tensor& y, const Tensor& delta, const Tensor& x, const Tensor& w_a, const Tensor& w_b,
+                        const Tensor& start_indicies, const Tensor& lora_ranks, const Tensor& loc_indicies,
+                        const Tensor& indicies, int64_t qkvo, const Tensor& lora_scales, const py::object& plan) {
+  SL_CHECK_INPUT(x);
+  SL_CHECK_DIM(2, x);
+  SL_CHECK_INPUT(w_a);
+  SL_CHECK_DIM(3, w_a);
+  SL_CHECK_INPUT(w_b);
+  SL_CHECK_DIM(3, w_b);
+  check_tables(start_indicies, lora_ranks, loc_indicies, indicies);
+  check_scales(lora_scales, start_indicies);
+  const int64_t batch = x.size(0), h_in = x.size(1);
+  const at::ScalarType dt = x.scalar_type();
+  check_rows_2d(delta, "delta", batch, -1, dt);
+  check_rows_2d(y, "y", batch, -1, dt);
+  SL_CHECK_EQ(indicies.size(0), x.size(0));
+  const int64_t d_cols = delta.size(1), h_out = y.size(1);
+  const bool dt_ok = (dt == at::kHalf || dt == at::kBFloat16) && w_a.scalar_type() == dt && w_b.scalar_type() == dt;
+  TORCH_CHECK(dt_ok && h_in < 65536 && h_out < 65536, "No suitable kernel. h_in=", h_in, " h_out=", h_out, " dtype=", dt);
+  TORCH_CHECK(w_a.sizes() == w_b.sizes(), "w_a and w_b must be pools of one shape (they share page ids)");
+  const int64_t page_elems = w_a.size(1) * w_a.size(2), n_pages = w_a.size(0);
+  const slora_tables t = tables_of(start_indicies, lora_ranks, loc_indicies);
+  const int code = dtype_code(x, "x"), sc = dtype_code(lora_scales, "lora_scales");
+  void* stream = stream_of(x);
+  const std::shared_ptr<BgmvPlan> p =
+      resolve_plan(plan, start_indicies, lora_ranks, loc_indicies, indicies, d_cols, n_pages, stream, batch);
+  const int64_t* bins = indicies.data_ptr<int64_t>();
+  int rc;
+  if (p && d_cols % 8 == 0) {
+    rc = slora_bgmv_lora_planned(p->buf.data_ptr(), p->rank_cap, p->n_items, 1, y.data_ptr(), nullptr, nullptr,
+                                 delta.data_ptr(), nullptr, nullptr, x.data_ptr(), w_a.data_ptr(), w_b.data_ptr(), &t, bins,
+                                 lora_scales.data_ptr(), sc, batch, h_in, d_cols, h_out, 0, 0, page_elems, n_pages,
+                                 (int)qkvo, code, stream);
+  } else {
+    rc = slora_bgmv_shrink(delta.data_ptr(), x.data_ptr(), w_a.data_ptr(), &t, bins, batch, h_in, d_cols, page_elems,
+                           n_pages, (int)qkvo, code, stream);
+    if (rc == SLORA_OK)
+      rc = slora_bgmv_expand(y.data_ptr(), delta.data_ptr(), w_b.data_ptr(), &t, bins, lora_scales.data_ptr(), sc, batch,
+                             d_cols, h_out, page_elems, n_pages, (int)qkvo, code, stream);
+  }
+  TORCH_CHECK(rc != SLORA_ERR_UNSUPPORTED, "No suitable kernel. h_in=", h_in, " h_out=", h_out, " dtype=", dt);
+  check_rc(rc, "dispatch_bgmv_lora");
+}
+
+// The same for q, k and v in one launch (they share x).
+void dispatch_bgmv_qkv_lora(const Tensor& y_q, const Tensor& y_k, const Tensor& y_v, const Tensor& d_q, const Tensor& d_k,
+                            const Tensor& d_v, const Tensor& x, const Tensor& w_a, const Tensor& w_b,
+                            const Tensor& start_indicies, const Tensor& lora_ranks, const Tensor& loc_indicies,
+                            const Tensor& indicies, const Tensor& lora_scales, const py::object& plan) {
+  SL_CHECK_INPUT(x);
+  SL_CHECK_DIM(2, x);
+  SL_CHECK_INPUT(w_a);
+  SL_CHECK_DIM(3, w_a);
+  SL_CHECK_INPUT(w_b);
+  SL_CHECK_DIM(3, w_b);
+  check_tables(start_indicies, lora_ranks, loc_indicies, indicies);
+  check_scales(lora_scales, start_indicies);
+  const int64_t batch = x.size(0), h_in = x.size(1);
+  const at::ScalarType dt = x.scalar_type();
+  check_rows_2d(d_q, "d_q", batch, -1, dt);
+  const int64_t d_cols = d_q.size(1);
+  check_rows_2d(d_k, "d_k", batch, d_cols, dt);
+  check_rows_2d(d_v, "d_v", batch, d_cols, dt);
+  check_rows_2d(y_q, "y_q", batch, -1, dt);
+  check_rows_2d(y_k, "y_k", batch, -1, dt);
+  check_rows_2d(y_v, "y_v", batch, -1, dt);
+  SL_CHECK_EQ(indicies.size(0), x.size(0));
+  const bool dt_ok = (dt == at::kHalf || dt == at::kBFloat16) && w_a.scalar_type() == dt && w_b.scalar_type() == dt;
+  TORCH_CHECK(dt_ok, "No suitable kernel. h_in=", h_in, " h_out=", y_q.size(1), " dtype=", dt);
+  TORCH_CHECK(w_a.sizes() == w_b.sizes(), "w_a and w_b must be pools of one shape (they share page ids)");
+  const int64_t page_elems = w_a.size(1) * w_a.size(2), n_pages = w_a.size(0);
+  const slora_tables t = tables_of(start_indicies, lora_ranks, loc_indicies);
+  const int code = dtype_code(x, "x"), sc = dtype_code(lora_scales, "lora_scales");
+  void* stream = stream_of(x);
+  const std::shared_ptr<BgmvPlan> p =
+      resolve_plan(plan, start_indicies, lora_ranks, loc_indicies, indicies, d_cols, n_pages, stream, batch);
+  const int64_t* bins = indicies.data_ptr<int64_t>();
+  int rc;
+  if (p && d_cols % 8 == 0) {
+    rc = slora_bgmv_lora_planned(p->buf.data_ptr(), p->rank_cap, p->n_items, 3, y_q.data_ptr(), y_k.data_ptr(),
+                                 y_v.data_ptr(), d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), x.data_ptr(),
+                                 w_a.data_ptr(), w_b.data_ptr(), &t, bins, lora_scales.data_ptr(), sc, batch, h_in, d_cols,
+                                 y_q.size(1), y_k.size(1), y_v.size(1), page_elems, n_pages, 0, code, stream);
+  } else {
+    rc = slora_bgmv_shrink_qkv(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), x.data_ptr(), w_a.data_ptr(), &t, bins,
+                               batch, h_in, d_cols, page_elems, n_pages, code, stream);
+    if (rc == SLORA_OK)
+      rc = slora_bgmv_expand_qkv(y_q.data_ptr(), y_k.data_ptr(), y_v.data_ptr(), d_q.data_ptr(), d_k.data_ptr(),
+                                 d_v.data_ptr(), w_b.data_ptr(), &t, bins, lora_scales.data_ptr(), sc, batch, d_cols,
+                                 y_q.size(1), y_k.size(1), y_v.size(1), page_elems, n_pages, code, stream);
+  }
+  TORCH_CHECK(rc != SLORA_ERR_UNSUPPORTED, "No suitable kernel. h_in=", h_in, " h_out=", y_q.size(1), " dtype=", dt);
+  check_rc(rc, "dispatch_bgmv_qkv_lora");
+}
+
 // ---------------------------------------------------------------------------
 // prefill
 // ---------------------------------------------------------------------------
@@ -1024,6 +1121,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("dispatch_bgmv_qkv_expand", &dispatch_bgmv_qkv_expand, py::arg("y_q"), py::arg("y_k"), py::arg("y_v"),
         py::arg("x_q"), py::arg("x_k"), py::arg("x_v"), py::arg("w"), py::arg("start_indicies"), py::arg("lora_ranks"),
         py::arg("loc_indicies"), py::arg("indicies"), py::arg("lora_scales"), py::arg("plan") = py::none());
+  m.def("dispatch_bgmv_lora", &dispatch_bgmv_lora, py::arg("y"), py::arg("delta"), py::arg("x"), py::arg("w_a"),
+        py::arg("w_b"), py::arg("start_indicies"), py::arg("lora_ranks"), py::arg("loc_indicies"), py::arg("indicies"),
+        py::arg("qkvo"), py::arg("lora_scales"), py::arg("plan") = py::none());
+  m.def("dispatch_bgmv_qkv_lora", &dispatch_bgmv_qkv_lora, py::arg("y_q"), py::arg("y_k"), py::arg("y_v"), py::arg("d_q"),
+        py::arg("d_k"), py::arg("d_v"), py::arg("x"), py::arg("w_a"), py::arg("w_b"), py::arg("start_indicies"),
+        py::arg("lora_ranks"), py::arg("loc_indicies"), py::arg("indicies"), py::arg("lora_scales"),
+        py::arg("plan") = py::none());
   m.def("make_plan", &make_plan, py::arg("start_indicies"), py::arg("lora_ranks"), py::arg("loc_indicies"),
         py::arg("indicies"), py::arg("rank_cap"), py::arg("n_pages"), py::arg("readback") = true);
   m.def("rebuild_plan", &rebuild_plan, py::arg("plan"), py::arg("start_indicies"), py::arg("lora_ranks"),

@@ -29,7 +29,8 @@ except ImportError as e:  # pragma: no cover
                       "run `python s-lora_amd/build.py`") from e
 
 from ._kernels import (BgmvPlan, SgmmPlan, clear_plan_cache, clear_prefill_plan_cache,  # noqa: F401,E402
-                       dispatch_bgmv, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_shrink,
+                       dispatch_bgmv, dispatch_bgmv_lora, dispatch_bgmv_qkv_expand, dispatch_bgmv_qkv_lora,
+                       dispatch_bgmv_qkv_shrink,
                        lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_expand_qkv, lora_get_qkvo_fwd_shrink,
                        lora_get_qkvo_fwd_shrink_qkv, make_plan,
                        make_prefill_plan, plan_cache_stats, rebuild_plan, set_plan_cache_enabled)

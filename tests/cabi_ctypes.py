@@ -45,6 +45,8 @@ SIGNATURES = {
                                        _I, _I, _P]),
     "slora_bgmv_expand_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64, _I64,
                                        _I64, _I64, _I64, _I64, _I64, _I, _I, _P]),
+    "slora_bgmv_lora_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64, _I64,
+                                     _I64, _I64, _I64, _I64, _I64, _I64, _I, _I, _P]),
     "slora_sgmm_shrink": (_I, [_P, _P, _P, _TP, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _I64,
                                _I, _I, _P]),
     "slora_sgmm_plan_bytes": (_I64, []),
