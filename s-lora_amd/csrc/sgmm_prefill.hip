@@ -51,6 +51,8 @@ __device__ __forceinline__ int64_t seg_page(const SegTables& t, int64_t li) {
   return (uint64_t)page < (uint64_t)t.n_pages ? page : -1;
 }
 
+__device__ __forceinline__ bool aligned16_dev(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; }
+
 // a_loc entry `li` -> page id with the load outside any branch: an unwanted or
 // out-of-range index reads a_start[0] instead (there is at least one adapter
 // whenever a request reaches this point) and is rejected afterwards.  Callers
@@ -375,6 +377,253 @@ __device__ __forceinline__ void shrink_k_loop_qkv(const uint16_t* const (&xline)
   }
 }
 
+// ---------------------------------------------------------------------------
+// K loop fed through LDS (large batches)
+// ---------------------------------------------------------------------------
+// With every compute unit streaming, what a register-fed loop can keep in flight (64 KB per
+// compute unit at 324 registers per lane) is what bounds it.  Here the 64-k blocks of a tile --
+// 64 token rows of x and the 16-row units of weight rows of every projection -- travel from
+// memory straight into a ring of LDS stages (global_load_lds_dwordx4: no registers held while a
+// load is in flight), up to 128 KB per compute unit, and the MFMA fragments are read from
+// there.  The four wavefronts split the tile's OUTPUT (two row fragments x half of the units
+// each) instead of K, so every output is one chain of products over all of K and nothing is
+// summed across wavefronts.
+//
+// A wave-wide load fills one 1 KiB chunk of a stage: 8 rows x 128 bytes, lane i at slot i.
+// Which 16-byte piece of its row a lane fetches is its slot's column xor the row (within the
+// chunk), so that the later fragment reads -- 16 rows at one piece index -- fall on 8 different
+// 16-byte columns: no bank conflicts on either side (SQ_LDS_BANK_CONFLICT reads 0).
+constexpr int kShrRingBytes = 128 * 1024;
+
+template <int U>  // 16-row units of weight rows per block: projections x 16-column tiles of the rank
+struct ShrRing {
+  static constexpr int kLoads = 8 + 2 * U;        // chunks per stage: 8 of x, 2 per unit
+  static constexpr int kLpw = (kLoads + 3) / 4;   // loads a wavefront issues per stage
+  static constexpr int kStage = kLoads * 1024;    // bytes
+  static constexpr int kStages = kShrRingBytes / kStage < 8 ? kShrRingBytes / kStage : 8;
+  static constexpr int kUpw = (U + 1) / 2;        // units per wavefront column
+};
+
+// s_waitcnt for "at most n vector memory operations of this wavefront outstanding" (gfx9 encoding)
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  static_assert(N >= 0 && N < 64, "vmcnt is six bits");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// The compiler may not move LDS accesses across these: the barrier builtin alone says nothing
+// about memory, and __syncthreads() would wait for every outstanding load (the ring's included).
+__device__ __forceinline__ void ring_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+// LDS writes of this wavefront done (lgkmcnt(0), nothing else), then the barrier
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+constexpr int kShrOutPitch = kShrNB + 8;  // 16-bit entries per row of the output staging tile (rows stay 16-byte aligned)
+constexpr int kShrOutBytes = kShrTM * kShrOutPitch * 2;
+
+// One pass (64 rank columns from nb0) over ALL tiles of a part -- rows row_first .. + m_rows of one
+// request -- as one stream of 64-k blocks: the loads run kStages - 1 blocks ahead of the products
+// across tile boundaries, so the ring never drains between the tiles of a part.  A tile's sums go
+// through a staging tile in LDS (s_out, behind the ring) and leave as whole 16-byte pieces, the
+// columns behind the adapter's rank (up to max_rank) as zeros.
+template <typename T, int NPROJ, int NT>
+__device__ __forceinline__ void shrink_part_lds_pass(const SegShrinkArgs& p, unsigned char* ring, uint16_t* s_out,
+                                                     int64_t row_first, int m_rows, int r_eff, int64_t base_li,
+                                                     int rank, int nb0, int nb_cnt) {
+  constexpr int U = NPROJ * NT;
+  using R = ShrRing<U>;
+  constexpr int NU = R::kUpw;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const uint16_t* xg = reinterpret_cast<const uint16_t*>(p.x);
+  const uint16_t* wg = reinterpret_cast<const uint16_t*>(p.w);
+
+  // ---- what this lane fetches: the chunks wave, wave + 4, ... of every stage (a chunk past the
+  // last one repeats it: same data to the same place).  Chunks 0..7 are x (loads q = 0, 1 of every
+  // wavefront), the others weight rows, whose addresses do not change over the part.
+  const int crow = lane >> 3, piece = (lane & 7) ^ crow;
+  const uint16_t* src_w[R::kLpw];  // entries 0, 1 unused
+  int chunk[R::kLpw];
+  {
+    int64_t pg[R::kLpw];
+#pragma unroll
+    for (int q = 0; q < R::kLpw; ++q) {
+      int l = wave + 4 * q;
+      if (l >= R::kLoads) l = R::kLoads - 1;
+      chunk[q] = l;
+      const int a = l - 8, u = a >> 1, pj = u / NT, t = u - pj * NT;
+      const int j = nb0 + t * 16 + (a & 1) * 8 + crow;  // rank row (weight chunks)
+      pg[q] = seg_page_nobranch(p.t, base_li + (int64_t)pj * rank + j, q >= 2 && j < r_eff && p.t.n_loc > 0);
+    }
+#pragma unroll
+    for (int q = 0; q < R::kLpw; ++q)  // a row that does not exist reads pool page 0: its products only reach columns that are zeroed
+      src_w[q] = wg + (pg[q] >= 0 ? pg[q] : 0) * p.w_stride + piece * 8;
+  }
+  typedef __attribute__((address_space(3))) unsigned char* LdsBytes;
+  typedef const __attribute__((address_space(1))) void* GlobalPtr;
+  LdsBytes lds = (LdsBytes)ring;
+  const int nblk = p.h_in >> 6;
+  const int n_mt = (m_rows + kShrTM - 1) / kShrTM;
+
+  // the block the next load fetches: (i_tile, i_blk); its x rows (rows past the end of the part
+  // repeat the last one: their results are not stored)
+  int i_tile = 0, i_blk = 0;
+  const uint16_t* src_x[2];
+  auto x_rows_of = [&](int tile) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      int m = tile * kShrTM + chunk[q] * 8 + crow;
+      if (m >= m_rows) m = m_rows - 1;
+      src_x[q] = xg + (row_first + m) * p.x_stride + piece * 8;
+    }
+  };
+  x_rows_of(0);
+  auto issue = [&](int stage) {
+#pragma unroll
+    for (int q = 0; q < R::kLpw; ++q) {
+      // the LDS address of a chunk is the same in every lane (it travels in M0)
+      const int off = __builtin_amdgcn_readfirstlane(stage * R::kStage + chunk[q] * 1024);
+      const uint16_t* src = (q < 2 ? src_x[q] : src_w[q]) + (int64_t)i_blk * 64;
+      if (q < 2)  // x is read once: nontemporal, so that it does not push the weight rows out of L2
+        __builtin_amdgcn_global_load_lds((GlobalPtr)src, (__attribute__((address_space(3))) void*)(lds + off), 16, 0, 2);
+      else
+        __builtin_amdgcn_global_load_lds((GlobalPtr)src, (__attribute__((address_space(3))) void*)(lds + off), 16, 0, 0);
+    }
+    // advance; past the last block of the part the last block is fetched again, into a stage nobody reads
+    if (i_blk + 1 < nblk) {
+      ++i_blk;
+    } else if (i_tile + 1 < n_mt) {
+      ++i_tile;
+      i_blk = 0;
+      x_rows_of(i_tile);
+    }
+  };
+
+  // ---- fragment reads: lane (lr, lg) of K step s wants row lr, piece 4 s + lg of a 16-row unit
+  const int lr = lane & 15, lg = lane >> 4;
+  int frag_off[2];
+#pragma unroll
+  for (int sk = 0; sk < 2; ++sk) frag_off[sk] = (((lr >> 3) * 64) + (lr & 7) * 8 + ((4 * sk + lg) ^ (lr & 7))) * 16;
+  const int u0 = wn * NU;
+
+#pragma unroll
+  for (int b = 0; b < R::kStages - 1; ++b) issue(b);
+  int stage = 0, refill = R::kStages - 1;
+  for (int tile = 0; tile < n_mt; ++tile) {
+    f32x4 acc[2][NU];
+#pragma unroll
+    for (int fi = 0; fi < 2; ++fi)
+#pragma unroll
+      for (int ui = 0; ui < NU; ++ui) acc[fi][ui] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < nblk; ++b) {
+      // this wavefront's share of the block has landed; meet: everybody's has, and everybody is
+      // done with the block before, whose stage is refilled next
+      wait_vm<(R::kStages - 2) * R::kLpw>();
+      ring_barrier();
+      issue(refill);
+      LdsBytes base = lds + stage * R::kStage;
+#pragma unroll
+      for (int sk = 0; sk < 2; ++sk) {
+        u32x4 a[2];
+#pragma unroll
+        for (int fi = 0; fi < 2; ++fi)
+          a[fi] = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(base + (2 * (2 * wm + fi)) * 1024 +
+                                                                                    frag_off[sk]);
+#pragma unroll
+        for (int ui = 0; ui < NU; ++ui) {
+          int u = u0 + ui;
+          if (u >= U) u = U - 1;  // a unit past the last one is multiplied again and not stored
+          const u32x4 bfr = *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(base + (8 + 2 * u) * 1024 +
+                                                                                               frag_off[sk]);
+#pragma unroll
+          for (int fi = 0; fi < 2; ++fi) acc[fi][ui] = mfma16<T>(a[fi], bfr, acc[fi][ui]);
+        }
+      }
+      stage = stage + 1 == R::kStages ? 0 : stage + 1;
+      refill = refill + 1 == R::kStages ? 0 : refill + 1;
+    }
+    // ---- the tile's sums: lane holds column lr, rows 4 lg + i of fragment (2 wm + fi), unit u0 + ui.
+    // (s_out is free: whoever read it for the tile before has passed this tile's barriers since)
+    const int m_cnt = m_rows - tile * kShrTM < kShrTM ? m_rows - tile * kShrTM : kShrTM;
+#pragma unroll
+    for (int pj = 0; pj < NPROJ; ++pj) {
+#pragma unroll
+      for (int ui = 0; ui < NU; ++ui) {
+        const int u = u0 + ui;
+        if (u < U && u / NT == pj) {
+          const int c = (u - pj * NT) * 16 + lr;
+#pragma unroll
+          for (int fi = 0; fi < 2; ++fi)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              s_out[((2 * wm + fi) * 16 + 4 * lg + i) * kShrOutPitch + c] =
+                  T::from_float(nb0 + c < r_eff ? acc[fi][ui][i] : 0.f);
+        }
+      }
+      lds_barrier();
+      // rows of 8 columns (16 bytes) each; columns behind the adapter's tiles are zeros
+      uint16_t* og = reinterpret_cast<uint16_t*>(p.o[pj]);
+      const int64_t orow0 = row_first + (int64_t)tile * kShrTM;
+      if ((nb_cnt & 7) == 0 && (p.o_stride & 7) == 0 && (nb0 & 7) == 0 && aligned16_dev(og)) {
+        const int pieces = nb_cnt >> 3;
+        for (int idx = tid; idx < m_cnt * pieces; idx += kShrThreads) {
+          const int m = idx / pieces, c8 = (idx - m * pieces) * 8;
+          u32x4 v = zero16();
+          if (c8 < NT * 16) v = *reinterpret_cast<const u32x4*>(s_out + m * kShrOutPitch + c8);
+          *reinterpret_cast<u32x4*>(og + (orow0 + m) * p.o_stride + nb0 + c8) = v;
+        }
+      } else {
+        for (int idx = tid; idx < m_cnt * nb_cnt; idx += kShrThreads) {
+          const int m = idx / nb_cnt, c = idx - m * nb_cnt;
+          og[(orow0 + m) * p.o_stride + nb0 + c] = c < NT * 16 ? s_out[m * kShrOutPitch + c] : (uint16_t)0;
+        }
+      }
+      if (NPROJ > 1) lds_barrier();  // the staging tile is rewritten for the next projection
+    }
+  }
+  wait_vm<0>();  // the loads past the end
+  ring_barrier();  // the ring and the staging tile are free again
+}
+
+// A part through the LDS ring: per pass of 64 rank columns the 16-column tiles that hold columns
+// of the adapter are multiplied; a pass behind the adapter's rank only writes zeros.
+template <typename T, int NPROJ>
+__device__ __forceinline__ void shrink_part_lds(const SegShrinkArgs& p, unsigned char* ring, int64_t row_first,
+                                                int m_rows, int r_eff, int64_t base_li, int rank) {
+  uint16_t* s_out = reinterpret_cast<uint16_t*>(ring + kShrRingBytes);
+  for (int nb0 = 0; nb0 < p.max_rank; nb0 += kShrNB) {
+    const int nb_cnt = p.max_rank - nb0 < kShrNB ? p.max_rank - nb0 : kShrNB;
+    const int n_tiles = (r_eff - nb0 + 15) >> 4 < 4 ? (r_eff - nb0 + 15) >> 4 : 4;
+    switch (n_tiles > 0 ? n_tiles : 0) {
+      case 1: shrink_part_lds_pass<T, NPROJ, 1>(p, ring, s_out, row_first, m_rows, r_eff, base_li, rank, nb0, nb_cnt); break;
+      case 2: shrink_part_lds_pass<T, NPROJ, 2>(p, ring, s_out, row_first, m_rows, r_eff, base_li, rank, nb0, nb_cnt); break;
+      case 3: shrink_part_lds_pass<T, NPROJ, 3>(p, ring, s_out, row_first, m_rows, r_eff, base_li, rank, nb0, nb_cnt); break;
+      case 4: shrink_part_lds_pass<T, NPROJ, 4>(p, ring, s_out, row_first, m_rows, r_eff, base_li, rank, nb0, nb_cnt); break;
+      default: {
+        // no column of the adapter in this pass: zeros
+#pragma unroll
+        for (int pj = 0; pj < NPROJ; ++pj) {
+          uint16_t* og = reinterpret_cast<uint16_t*>(p.o[pj]);
+          for (int idx = threadIdx.x; idx < m_rows * nb_cnt; idx += kShrThreads) {
+            const int m = idx / nb_cnt, c = idx - m * nb_cnt;
+            og[(row_first + m) * p.o_stride + nb0 + c] = 0;
+          }
+        }
+        break;
+      }
+    }
+  }
+}
+
 // One tile: token rows row_first .. row_first + m_cnt (m_cnt <= kShrTM) of a request
 // whose weight rows start at a_loc[base_li]; of every 64 rank columns the 16-column
 // tiles t with t % p.col_split == cg.  All threads of the workgroup call it together;
@@ -576,8 +825,13 @@ __device__ __forceinline__ int shrink_chunks_needed(int units, int r_eff, uint32
 // read the same weight rows, share an L2) and every workgroup the same cost,
 // whatever the mix of request lengths and ranks.  A workgroup owns the units
 // whose start falls into its part and walks them as tiles of up to kShrMF units.
-template <typename T, int NPROJ, bool DEEP>
-__global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegShrinkArgs p) {
+// RING: the K loop fed through LDS (shrink_part_lds; launches whose every workgroup has whole tiles
+// and whole 64-k blocks), otherwise from registers (shrink_tile), DEEP with three blocks in flight
+// per wavefront.  The ring kernels need half the register file at most, and with no more than 256
+// registers a wavefront the matrix instructions accumulate in ordinary registers instead of being
+// copied in and out of the accumulation registers around every block.
+template <typename T, int NPROJ, bool DEEP, bool RING>
+__global__ __launch_bounds__(kShrThreads, RING ? 2 : 1) void sgmm_shrink_kernel(const SegShrinkArgs p) {
   extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
   __shared__ int64_t s_wave[kShrWaves];
   __shared__ int s_row0[kShrChunk], s_rows[kShrChunk], s_ub[kShrChunk], s_ue[kShrChunk], s_rank[kShrChunk];
@@ -759,7 +1013,15 @@ __global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_kernel(const SegSh
       const int64_t bl = s_base[j];
       const int64_t base_li =
           (int64_t)(((uint64_t)(uint32_t)uni((int)((uint64_t)bl >> 32)) << 32) | (uint32_t)uni((int)(uint32_t)bl));
-      for (int u = u0; u < u1; u += kShrMF) {
+      if constexpr (RING) {
+        // all tiles of the request's share as one stream of blocks (the launcher picks this
+        // instantiation only for layouts the vector path reads)
+        const int m0 = u0 * kShrUnit, m_end = u1 * kShrUnit < rows ? u1 * kShrUnit : rows;
+        if (m_end > m0)
+          shrink_part_lds<T, NPROJ>(p, reinterpret_cast<unsigned char*>(s_part), (int64_t)rw0 + m0, m_end - m0, r_eff,
+                                    base_li, rj);
+      }
+      for (int u = u0; !RING && u < u1; u += kShrMF) {
         const int m0 = u * kShrUnit;
         int m_end = (u + kShrMF < u1 ? u + kShrMF : u1) * kShrUnit;
         if (m_end > rows) m_end = rows;
@@ -864,22 +1126,32 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_plan_kernel(int* plan, SegTa
   }
 }
 
-template <typename T, int NPROJ, bool DEEP>
-__global__ __launch_bounds__(kShrThreads, 1) void sgmm_shrink_planned_kernel(const SegShrinkArgs p, const int* plan) {
-  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd]
+template <typename T, int NPROJ, bool DEEP, bool RING>
+__global__ __launch_bounds__(kShrThreads, RING ? 2 : 1) void sgmm_shrink_planned_kernel(const SegShrinkArgs p,
+                                                                                        const int* plan) {
+  extern __shared__ float s_part[];  // [kShrWaves][kShrTM][kShrLd], or the ring and its staging tile
   const int slot = (int)(blockIdx.x & 7) * ((int)gridDim.x >> 3) + (int)(blockIdx.x >> 3);
   const int parts = (int)gridDim.x / p.col_split;
-  const int part = slot / p.col_split, cg = slot - part * p.col_split;
-  // header and record of this part in one group of scalar loads
-  const int* rec = plan + kSegPlanHeaderWords + part * kSegPartWords;
-  int magic = plan[SP_MAGIC], n_parts = plan[SP_PARTS], split = plan[SP_SPLIT];
+  // (an integer division runs on the vector unit: say that its result is the same in every lane)
+  const int part = __builtin_amdgcn_readfirstlane(slot / p.col_split), cg = slot - part * p.col_split;
+  // header and record of this part in one group of scalar loads (the plan does not change while
+  // this kernel runs: reading it through the constant address space keeps the loads scalar
+  // whatever else the kernel writes)
+  typedef const int __attribute__((address_space(4))) * ConstWords;
+  ConstWords head = (ConstWords)plan;
+  ConstWords rec = head + kSegPlanHeaderWords + part * kSegPartWords;
+  int magic = head[SP_MAGIC], n_parts = head[SP_PARTS], split = head[SP_SPLIT];
   int row_first = rec[PT_ROW], m_rows = rec[PT_ROWS], r = rec[PT_RANK], lo = rec[PT_START_LO], hi = rec[PT_START_HI];
   asm volatile("" : "+s"(magic), "+s"(n_parts), "+s"(split), "+s"(row_first), "+s"(m_rows), "+s"(r), "+s"(lo), "+s"(hi));
   if (magic != kSegPlanMagic || n_parts != parts || split != p.col_split) return;  // not a plan of this launch shape
   if (m_rows <= 0 || row_first < 0 || m_rows > p.t.n_tokens - row_first) return;
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   const int64_t base_li = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo) + (int64_t)r * p.qkvo;
-  for (int m0 = 0; m0 < m_rows; m0 += kShrTM) {
+  if constexpr (RING) {  // all tiles of the part as one stream of blocks
+    shrink_part_lds<T, NPROJ>(p, reinterpret_cast<unsigned char*>(s_part), row_first, m_rows, r_eff, base_li, r);
+    return;
+  }
+  for (int m0 = 0; !RING && m0 < m_rows; m0 += kShrTM) {
     const int m_cnt = m_rows - m0 < kShrTM ? m_rows - m0 : kShrTM;
     if (!p.vec_ok) {
       if (cg == 0)
@@ -1396,24 +1668,37 @@ bool shrink_plan_usable(int64_t n_requests, int64_t m_tiles, int64_t grid, int c
 
 // DEEP: the instantiation whose single-projection K loop keeps three blocks in flight (for
 // launches with few workgroups, see shrink_k_loop_ring)
+template <typename T, int NPROJ, bool DEEP, bool RING>
+int launch_seg_shrink_kernel(const SegShrinkArgs& q, const int* plan, int64_t grid, size_t lds, hipStream_t stream) {
+  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ, DEEP, RING>)
+                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ, DEEP, RING>);
+  static PerDeviceOnce once[2];
+  if (!raise_dynamic_lds(kernel, (int)lds, once[plan != nullptr])) return SLORA_ERR_LAUNCH;
+  if (plan != nullptr)
+    hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ, DEEP, RING>), dim3((uint32_t)grid), dim3(kShrThreads), lds,
+                       stream, q, plan);
+  else
+    hipLaunchKernelGGL((sgmm_shrink_kernel<T, NPROJ, DEEP, RING>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream,
+                       q);
+  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+}
+
 template <typename T, int NPROJ, bool DEEP>
 int launch_seg_shrink(const SegShrinkArgs& p, const int* plan, hipStream_t stream) {
-  const size_t lds = sizeof(float) * kShrWaves * kShrTM * kShrLd;
   int64_t grid = 0;
   SegShrinkArgs q = p;
   shrink_geometry(p.t.n_tokens, p.t.n_requests, p.m_tiles, p.max_rank, grid, q.col_split);
   if (grid <= 0) return SLORA_OK;
   if (plan != nullptr && !shrink_plan_usable(p.t.n_requests, p.m_tiles, grid, q.col_split)) return SLORA_ERR_BAD_SHAPE;
-  const void* kernel = plan != nullptr ? reinterpret_cast<const void*>(sgmm_shrink_planned_kernel<T, NPROJ, DEEP>)
-                                       : reinterpret_cast<const void*>(sgmm_shrink_kernel<T, NPROJ, DEEP>);
-  static PerDeviceOnce once[2];
-  if (!raise_dynamic_lds(kernel, (int)lds, once[plan != nullptr])) return SLORA_ERR_LAUNCH;
-  if (plan != nullptr)
-    hipLaunchKernelGGL((sgmm_shrink_planned_kernel<T, NPROJ, DEEP>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q,
-                       plan);
-  else
-    hipLaunchKernelGGL((sgmm_shrink_kernel<T, NPROJ, DEEP>), dim3((uint32_t)grid), dim3(kShrThreads), lds, stream, q);
-  return hipGetLastError() == hipSuccess ? SLORA_OK : SLORA_ERR_LAUNCH;
+  // Large batches (every compute unit has a tile of its own) with whole 64-k blocks: the K loop through
+  // the LDS ring.  Beyond kShrDeepTokens for q/k/v too, so that the fused launch stays bit for bit the
+  // three calls.
+  if constexpr (!DEEP) {
+    const bool ring = p.t.n_tokens > kShrDeepTokens && q.col_split == 1 && p.vec_ok && (p.h_in & 63) == 0 && p.h_in >= 64;
+    if (ring)
+      return launch_seg_shrink_kernel<T, NPROJ, false, true>(q, plan, grid, kShrRingBytes + kShrOutBytes, stream);
+  }
+  return launch_seg_shrink_kernel<T, NPROJ, DEEP, false>(q, plan, grid, sizeof(float) * kShrWaves * kShrTM * kShrLd, stream);
 }
 
 template <typename T, int KS, int NPROJ>
