@@ -1636,7 +1636,8 @@ int fill_seg_tables(SegTables& t, const slora_tables* in, const int32_t* b_start
 // rows while each of the others streams all weight rows of its tile, so the rank columns of
 // a tile are then shared by 2 or 4 workgroups: the split with the least estimated time of
 // the slowest workgroup (14.2 us + per tile 0.2 us per weight row it reads + 0.177 us per
-// row; further tiles 6.7 us each).  grid = 0: nothing to do.
+// row; further tiles 6.7 us each).  Batches beyond kShrDeepTokens are not split (they take the
+// kernels that stream whole tiles through LDS).  grid = 0: nothing to do.
 void shrink_geometry(int64_t n_tokens, int64_t n_requests, int64_t m_tiles, int64_t max_rank, int64_t& grid, int& cs) {
   grid = 0;
   cs = 1;
@@ -1647,6 +1648,7 @@ void shrink_geometry(int64_t n_tokens, int64_t n_requests, int64_t m_tiles, int6
   float best = 0.f;
   for (int c = 1; c <= 4; c *= 2) {
     if (c > 1 && max_rank < 16 * c) break;  // fewer 16-column tiles than workgroups to share them
+    if (c > 1 && n_tokens > kShrDeepTokens) break;  // such batches stream through the LDS ring, whole tiles per workgroup
     const int64_t row_parts = kShrMaxGrid / c;
     int64_t rows = (n_tokens + row_parts - 1) / row_parts;
     rows = (rows + kShrUnit - 1) / kShrUnit * kShrUnit;
