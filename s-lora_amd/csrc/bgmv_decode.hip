@@ -32,7 +32,7 @@ namespace {
 // NV: the straight-line path of this instantiation holds pages of up to 512 * NV elements
 // (8: hidden <= 4096; larger ones cost registers, so the host picks the smallest that fits)
 template <typename T, bool PLANNED, int NV>
-__global__ __launch_bounds__(256) void bgmv_shrink_kernel(const ShrinkArgs p) {
+__global__ __launch_bounds__(256, NV == 8 ? 4 : 1) void bgmv_shrink_kernel(const ShrinkArgs p) {
   extern __shared__ u32x4 s_x[];  // [lds_tt][h_in / 8]
   int unit = (int)blockIdx.x;
   Item it;
