@@ -154,7 +154,8 @@ def make_step(w, bufs, mode, keep_plan=False):
         return sweep
 
     nv = next((n for n in (8, 10, 12, 16) if w.hidden <= 512 * n), 8)  # the instantiation the library picks
-    sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}, {nv}>", f"bgmv_expand_kernel<{ty}, %d, {pl}>"
+    nv_e = nv if planned else 8   # the stateless expand keeps the 4096-element pass
+    sk, ek = f"bgmv_shrink_kernel<{ty}, {pl}, {nv}>", f"bgmv_expand_kernel<{ty}, %d, {pl}, {nv_e}>"
     if one_launch:
         lk = f"bgmv_lora_kernel<{ty}, %d, {nv}>"
         families = {
@@ -525,10 +526,11 @@ def measure_prefill(args, torch, device, w=None, seg=None):
     ms_step_fused = time_region(wrap(step_fused), reps, args.warmup, torch)
     kernels = {}
     flops1 = seg.flops(w, H)
+    ring = "true" if T > 4096 and H % 64 == 0 else "false"   # the instantiation that streams through LDS
     for label, sweep, kname, nbytes, flops in (
-            ("shrink", shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 1, {'true' if T <= 4096 else 'false'}>",
+            ("shrink", shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 1, {'true' if T <= 4096 else 'false'}, {ring}>",
              seg.shrink_bytes(w), flops1),
-            ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3, false>",
+            ("qkv_shrink", qkv_shrink_sweep, f"sgmm_shrink_planned_kernel<{ty}, 3, false, {ring}>",
              3 * seg.shrink_bytes(w) - 2 * T * H * 2, 3 * flops1),
             ("expand", expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}, 1>", seg.expand_bytes(w, H), flops1),
             ("qkv_expand", qkv_expand_sweep, f"sgmm_expand_walk_kernel<{ty}, {ks}, 3>", 3 * seg.expand_bytes(w, H),

@@ -403,6 +403,55 @@ def test_prefill_qkv_shrink_gives_the_three_calls_bits(gpu, dtype, hidden, ranks
     np.testing.assert_allclose(host(single[1][:T, :R]), d_ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("hidden,ranks,n_req,lo,hi,sort,x_pad,o_off", [
+    (256, [8, 16, 32, 64], 60, 60, 110, True, 0, 0),      # whole and partial 64-row tiles of every tile count
+    (512, [128, 24, 40], 50, 80, 130, False, 0, 0),       # two passes over the rank; ranks that end inside a 16-column tile
+    (256, [64, 8], 70, 1, 150, False, 64, 8),             # strided x, output columns at an aligned offset of a wider buffer
+    (128, [32, 16], 40, 100, 140, True, 8, 4),            # output rows that are not 16-byte aligned: element-wise stores
+    (128, [64, 16], 20, 900, 1100, True, 0, 0),           # more than 64 rows per workgroup: several tiles in one stream of blocks
+])
+def test_prefill_shrink_above_4096_tokens(gpu, dtype, hidden, ranks, n_req, lo, hi, sort, x_pad, o_off):
+    """Batches of more than 4096 tokens take the kernels whose K loop streams through LDS (whole
+    64-k blocks, 64-row tiles, the wavefronts splitting the outputs): single projection and
+    q/k/v in one launch against the oracle at rtol 1e-2 / atol 1e-3, the fused launch bit for bit
+    the three calls, with and without a plan; columns outside [0, max_rank) of a wider output
+    buffer and rows of no request keep what they held."""
+    from slora_hip import lora_get_qkvo_fwd_shrink, lora_get_qkvo_fwd_shrink_qkv
+    c = seg_case(2000 + hidden + n_req, hidden, ranks, n_req, lo, hi, dtype, sort=sort)
+    assert c.batch > 4096
+    g = GpuCase(c, gpu)
+    start, lens, ids, max_len = _shrink_args(c, g, gpu)
+    R = (max(ranks) + 7) // 8 * 8
+    T = c.batch
+    w_a = g.key.view(c.n_pages, c.page_elems)
+    xb = torch.zeros((T + 2, hidden + x_pad), dtype=g.tdt, device=gpu)
+    xb[:T, :hidden] = g.x
+    x = xb[:, :hidden]
+    t = (g.a_loc, g.a_start, g.a_len, start, lens, ids)
+    outs = {}
+    for how in (False, None):
+        single = []
+        for p in range(3):
+            ob = torch.full((T + 2, R + 16), 7.0, dtype=g.tdt, device=gpu)
+            lora_get_qkvo_fwd_shrink(x, w_a, ob[:, o_off:o_off + R], *t, hidden, p, R, max_len, plan=how)
+            single.append(ob)
+        fused = [torch.full((T + 2, R + 16), 7.0, dtype=g.tdt, device=gpu) for _ in range(3)]
+        lora_get_qkvo_fwd_shrink_qkv(x, w_a, *[f[:, o_off:o_off + R] for f in fused], *t, hidden, R, max_len, plan=how)
+        torch.cuda.synchronize()
+        for p in range(3):
+            assert torch.equal(fused[p], single[p]), (p, how)
+        outs[how] = single
+    for p in range(3):
+        assert torch.equal(outs[False][p], outs[None][p]), p
+        ob = outs[None][p]
+        d_ref = O.ref_prefill_shrink(np.full((T, R), 7.0, np.float32), c.x, c.key, c.a_loc, c.a_start, c.a_len, c.start,
+                                     c.lens, c.ids, p, R, c.dtype)
+        np.testing.assert_allclose(host(ob[:T, o_off:o_off + R]), d_ref, rtol=RTOL, atol=ATOL)
+        keep = torch.full((1,), 7.0, dtype=g.tdt, device=gpu)
+        assert torch.all(ob[:, :o_off] == keep) and torch.all(ob[:, o_off + R:] == keep) and torch.all(ob[T:] == keep)
+
+
 def test_prefill_qkv_shrink_rejects_mismatched_outputs(gpu):
     from slora_hip import lora_get_qkvo_fwd_shrink_qkv
     c = seg_case(33, 256, [16, 8], 6, 1, 50, "f16")
