@@ -40,7 +40,7 @@ extern "C" {
  *   2.0 (200): slora_bgmv_lora_planned (shrink and expand in one launch) has a new signature and a
  *              new plan layout behind it -- the 1.0 form was removed in 1.1 without a major bump,
  *              which this number corrects; plans hold hand-over counters (slora_bgmv_plan_bytes
- *              grew); + slora_pool_page_xor.
+ *              grew); + slora_pool_page_xor, slora_plan_status.
  *   1.2 (102): + slora_sgmm_expand_qkv.
  *   1.1 (101): + slora_sgmm_shrink_qkv, slora_pool_page_checksums, slora_pool_pack_transposed,
  *              slora_pool_alloc_contiguous_static; - slora_bgmv_lora_planned. */
@@ -146,6 +146,17 @@ SLORA_API int64_t slora_bgmv_plan_bytes(int64_t batch, int64_t rank_cap);
 SLORA_API int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_tables* tables,
                                     const int64_t* bins, int64_t batch, int64_t rank_cap,
                                     int64_t n_pages, void* stream);
+
+/* Status word of a plan (of slora_bgmv_plan_build or slora_sgmm_plan_build), copied to the host;
+ * WAITS for the work queued on `stream`.  0 after a build.  Bit 0: a launch was given this plan
+ * with another batch size, rank cap or launch shape than the plan was built for -- such a launch
+ * does nothing (the outputs keep their values) and leaves this mark instead of an error code,
+ * because only the device can tell.  Bit 1: a hand-over inside slora_bgmv_lora_planned was
+ * abandoned after its poll limit.  The mark covers a wrong plan in a large enough buffer only: a
+ * planned launch reads its item records before it has seen the header, so the buffer it is given
+ * must hold slora_bgmv_plan_bytes(batch, rank_cap) bytes for the batch and rank cap OF THE LAUNCH,
+ * whatever the plan in it was built for.  No counterpart in the reference. */
+SLORA_API int slora_plan_status(const void* plan, int* status, void* stream);
 
 /* slora_bgmv_shrink / slora_bgmv_shrink_qkv with a plan.  nproj = 1: y0 and
  * qkvo as in slora_bgmv_shrink; nproj = 3: y0,y1,y2 = q,k,v and qkvo = 0.

@@ -237,6 +237,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_kernel(int* __restrict
     plan[PH_TT] = kTT;
     plan[PH_RANKCAP] = rank_cap;
     plan[PH_NRUNS] = n_runs;
+    plan[PH_STATUS] = 0;
   }
 }
 
@@ -403,6 +404,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_fast_kernel(int* __res
     plan[PH_TT] = kTT;
     plan[PH_RANKCAP] = rank_cap;
     plan[PH_NRUNS] = n_runs;
+    plan[PH_STATUS] = 0;
   }
 }
 
@@ -610,6 +612,7 @@ __global__ __launch_bounds__(kPlanThreads) void bgmv_plan_sort_kernel(int* __res
     plan[PH_TT] = kTT;
     plan[PH_RANKCAP] = rank_cap;
     plan[PH_NRUNS] = n_runs;
+    plan[PH_STATUS] = 0;
   }
 }
 

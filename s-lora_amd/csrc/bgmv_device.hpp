@@ -46,7 +46,10 @@ constexpr int kSyncHeader = 4;          // [0]: set when a hand-over gave up wai
 enum { SY_TIMEOUT = 0 };
 constexpr int kPlanHeaderWords = 16;
 constexpr int kItemWords = 48;
-enum { PH_MAGIC = 0, PH_NITEMS = 1, PH_MAXRANK = 2, PH_BATCH = 3, PH_TT = 4, PH_RANKCAP = 5, PH_NRUNS = 6 };
+enum { PH_MAGIC = 0, PH_NITEMS = 1, PH_MAXRANK = 2, PH_BATCH = 3, PH_TT = 4, PH_RANKCAP = 5, PH_NRUNS = 6, PH_STATUS = 7 };
+// PH_STATUS (0 after a build; read back with slora_plan_status): bit 0 = a launch named another batch size
+// or rank cap than the plan was built for and did nothing; bit 1 = a hand-over of the one-launch LoRA gave up
+enum { kPlanStatusMismatch = 1, kPlanStatusTimeout = 2 };
 enum { IT_ADAPTER = 0, IT_RANK = 1, IT_NTOK = 2, IT_J0 = 3, IT_TOK = 4, IT_PAGES = 8, IT_BASE = 40, IT_MORE = 42 };
 
 struct Item {
@@ -144,8 +147,8 @@ __device__ __forceinline__ void discover_run(const Tables& t, int batch, int b, 
 // read up front and pinned in scalar registers before the first branch, so the
 // compiler cannot sink the loads below the early exits: header check, record
 // and page ids are ONE round trip of independent scalar loads.
-__device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx, int pp, int jr0, int jr1, Item& it,
-                                          int& page0, int& page1) {
+__device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx, int pp, int jr0, int jr1, int batch,
+                                          int rank_cap, Item& it, int& page0, int& page1) {
   // The header and the records do not change while a kernel that reads them runs
   // (the counters behind them do, through another pointer): reading them through
   // the constant address space keeps these loads scalar whatever else the kernel
@@ -153,7 +156,7 @@ __device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx,
   typedef const int __attribute__((address_space(4))) * ConstWords;
   ConstWords head = (ConstWords)plan;
   ConstWords rec = head + kPlanHeaderWords + (int64_t)idx * kItemWords;
-  int magic = head[PH_MAGIC], n_items = head[PH_NITEMS];
+  int magic = head[PH_MAGIC], n_items = head[PH_NITEMS], plan_batch = head[PH_BATCH], plan_cap = head[PH_RANKCAP];
   int a = rec[IT_ADAPTER], r = rec[IT_RANK], n_tok = rec[IT_NTOK], j0 = rec[IT_J0];
   int t0 = rec[IT_TOK + 0], t1 = rec[IT_TOK + 1], t2 = rec[IT_TOK + 2], t3 = rec[IT_TOK + 3];
   int more = rec[IT_MORE];
@@ -167,8 +170,11 @@ __device__ __forceinline__ void load_item(const int* __restrict__ plan, int idx,
   it.tok[1] = t1;
   it.tok[2] = t2;
   it.tok[3] = t3;
-  const bool ok = (magic == kPlanMagic) & (idx < n_items);
-  it.plan_items = magic == kPlanMagic ? n_items : 0;
+  // a plan of another batch or rank cap lists other tokens and rows: nothing is done, and the plan says so
+  const bool mine = (magic == kPlanMagic) & (plan_batch == batch) & (plan_cap == rank_cap);
+  if ((magic == kPlanMagic) & !mine & (idx == 0) & (threadIdx.x == 0)) const_cast<int*>(plan)[PH_STATUS] = kPlanStatusMismatch;
+  const bool ok = mine & (idx < n_items);
+  it.plan_items = mine ? n_items : 0;
   it.a = a;
   it.r = r;
   it.n_tok = ok ? n_tok : 0;
@@ -199,6 +205,7 @@ struct ShrinkArgs {
   Tables t;
   int64_t page_elems;
   int batch, h_in, y_cols, qkvo0, blocks, lds_tt;
+  int rank_cap;  // of the plan the caller names (planned launches)
   int strided;  // planned launch with fewer workgroups than the plan may have items (see planned_grid)
 };
 
@@ -306,7 +313,7 @@ __device__ __forceinline__ int shrink_body(const ShrinkArgs& p, int unit, int pr
   const int* rec = PLANNED ? p.plan + kPlanHeaderWords + (int64_t)unit * kItemWords : nullptr;
   int plan_pg0 = -1, plan_pg1 = -1;
   if (PLANNED) {
-    load_item(p.plan, unit, p.qkvo0 + proj, wave, wave + 4, it, plan_pg0, plan_pg1);
+    load_item(p.plan, unit, p.qkvo0 + proj, wave, wave + 4, p.batch, p.rank_cap, it, plan_pg0, plan_pg1);
   } else {
     const int b = unit / p.blocks;
     discover_run(p.t, p.batch, b, it);
@@ -462,6 +469,7 @@ struct ExpandArgs {
   int64_t page_elems;
   int scales_dtype;
   int batch, x_cols, qkvo0, blocks, y_aligned;
+  int rank_cap;  // of the plan the caller names (planned launches)
   int interleave;  // one-dimensional grid: the workgroups of an item follow each other (see bgmv_expand_kernel)
   int strided;     // planned launch with fewer workgroups than the plan may have items (see planned_grid)
   int n_units;     // items (planned) or token blocks (stateless) of the launch
@@ -758,7 +766,7 @@ __device__ __forceinline__ int expand_body(const ExpandArgs& p, int unit, int su
   Item it;
   int plan_pg = -1, plan_pg_unused = -1;
   if (PLANNED) {
-    load_item(p.plan, unit, p.qkvo0 + proj, jr, jr, it, plan_pg, plan_pg_unused);
+    load_item(p.plan, unit, p.qkvo0 + proj, jr, jr, p.batch, p.rank_cap, it, plan_pg, plan_pg_unused);
   } else {
     const int b = unit / p.blocks;
     discover_run(p.t, p.batch, b, it);
@@ -893,6 +901,7 @@ int shrink_prepare(const void* plan, int64_t n_items, int64_t rank_cap, void* co
   p.y_cols = (int)y_cols;
   p.qkvo0 = qkvo0;
   p.blocks = (int)((y_cols + kRB - 1) / kRB);
+  p.rank_cap = (int)rank_cap;
   p.strided = 0;
   grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap, p.strided) : batch * p.blocks;
   return SLORA_OK;
@@ -955,6 +964,7 @@ int expand_prepare(const void* plan, int64_t n_items, int64_t rank_cap, void* co
   // stateless: the rank is only known on the device; the grid covers the pages of a rank
   // up to the delta width (an adapter uses min(rank, ceil(h_out*rank/page_elems)) pages)
   p.blocks = (int)((x_cols + kRB - 1) / kRB);
+  p.rank_cap = (int)rank_cap;
   p.strided = 0;
   grid = plan != nullptr ? planned_grid(n_items, batch, rank_cap, p.strided) : batch * p.blocks;
   return SLORA_OK;

@@ -68,7 +68,11 @@ __device__ __forceinline__ void lora_wait(const LoraArgs& p, const Item& it, int
       int spins = 0;
       while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target < 0) {
         if (++spins > p.spin_limit) {  // never expected; leaves a mark instead of waiting for ever
-          if (threadIdx.x == 0) p.sync[SY_TIMEOUT] = 1;
+          if (threadIdx.x == 0) {
+            p.sync[SY_TIMEOUT] = 1;
+            __hip_atomic_fetch_or(const_cast<int*>(p.s.plan) + PH_STATUS, kPlanStatusTimeout, __ATOMIC_RELAXED,
+                                  __HIP_MEMORY_SCOPE_AGENT);
+          }
           break;
         }
         __builtin_amdgcn_s_sleep(4);

@@ -1,4 +1,6 @@
 // Version and error strings of the C ABI.
+#include <hip/hip_runtime.h>
+
 #include "slora_hip.h"
 
 extern "C" {
@@ -17,6 +19,18 @@ const char* slora_strerror(int code) {
     case SLORA_ERR_TOO_LARGE: return "size exceeds the fixed capacity of this entry point (see its maximum in slora_hip.h)";
     default: return "unknown error";
   }
+}
+
+int slora_plan_status(const void* plan, int* status, void* stream) {
+  if (plan == nullptr || status == nullptr) return SLORA_ERR_NULL_POINTER;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  // word 7 of both plan headers
+  if (hipMemcpyAsync(status, static_cast<const int*>(plan) + 7, sizeof(int), hipMemcpyDeviceToHost, s) != hipSuccess ||
+      hipStreamSynchronize(s) != hipSuccess) {
+    (void)hipGetLastError();
+    return SLORA_ERR_LAUNCH;
+  }
+  return SLORA_OK;
 }
 
 }  // extern "C"

@@ -1050,7 +1050,7 @@ __global__ __launch_bounds__(kShrThreads, RING ? 2 : 1) void sgmm_shrink_kernel(
 constexpr int kSegPlanMagic = 0x53475031;
 constexpr int kSegPlanHeaderWords = 16;
 constexpr int kSegPartWords = 8;
-enum SegPlanHeader { SP_MAGIC = 0, SP_PARTS, SP_SPLIT, SP_NREQ, SP_NTOKENS, SP_MAXRANK, SP_ROWCAP };
+enum SegPlanHeader { SP_MAGIC = 0, SP_PARTS, SP_SPLIT, SP_NREQ, SP_NTOKENS, SP_MAXRANK, SP_ROWCAP, SP_STATUS };  // SP_STATUS: as PH_STATUS of the decode plan (word 7)
 enum SegPart { PT_ROW = 0, PT_ROWS, PT_RANK, PT_START_LO, PT_START_HI };
 
 // One workgroup.  Same scheme as the few-requests case of sgmm_shrink_kernel (request j
@@ -1123,6 +1123,7 @@ __global__ __launch_bounds__(kShrThreads) void sgmm_plan_kernel(int* plan, SegTa
     plan[SP_NTOKENS] = t.n_tokens;
     plan[SP_MAXRANK] = max_rank;
     plan[SP_ROWCAP] = row_cap;
+    plan[SP_STATUS] = 0;
   }
 }
 
@@ -1143,7 +1144,10 @@ __global__ __launch_bounds__(kShrThreads, RING ? 2 : 1) void sgmm_shrink_planned
   int magic = head[SP_MAGIC], n_parts = head[SP_PARTS], split = head[SP_SPLIT];
   int row_first = rec[PT_ROW], m_rows = rec[PT_ROWS], r = rec[PT_RANK], lo = rec[PT_START_LO], hi = rec[PT_START_HI];
   asm volatile("" : "+s"(magic), "+s"(n_parts), "+s"(split), "+s"(row_first), "+s"(m_rows), "+s"(r), "+s"(lo), "+s"(hi));
-  if (magic != kSegPlanMagic || n_parts != parts || split != p.col_split) return;  // not a plan of this launch shape
+  if (magic != kSegPlanMagic || n_parts != parts || split != p.col_split) {  // not a plan of this launch shape: nothing is done
+    if (magic == kSegPlanMagic && blockIdx.x == 0 && threadIdx.x == 0) const_cast<int*>(plan)[SP_STATUS] = 1;
+    return;
+  }
   if (m_rows <= 0 || row_first < 0 || m_rows > p.t.n_tokens - row_first) return;
   const int r_eff = r < p.max_rank ? r : p.max_rank;
   const int64_t base_li = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo) + (int64_t)r * p.qkvo;

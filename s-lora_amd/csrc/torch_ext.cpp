@@ -122,6 +122,13 @@ bool env_cache_default() {
 }
 bool g_cache_enabled = env_cache_default();
 
+// status word of a plan buffer, read back on the buffer's current stream
+int64_t plan_status_of(const Tensor& buf) {
+  int status = 0;
+  check_rc(slora_plan_status(buf.data_ptr(), &status, stream_of(buf)), "plan status");
+  return status;
+}
+
 // ---------------------------------------------------------------------------
 // decode plans
 // ---------------------------------------------------------------------------
@@ -1102,14 +1109,20 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
       .def_readonly("batch", &BgmvPlan::batch)
       .def_readwrite("n_items", &BgmvPlan::n_items)
       .def_readonly("max_rank", &BgmvPlan::max_rank)
-      .def_readonly("n_runs", &BgmvPlan::n_runs);
+      .def_readonly("n_runs", &BgmvPlan::n_runs)
+      .def("status", [](const BgmvPlan& pl) { return plan_status_of(pl.buf); },
+           "status word of the plan (waits for the current stream): 0, or bit 0 = a launch named another batch "
+           "size or rank cap and did nothing, bit 1 = a hand-over of the one-launch LoRA was abandoned");
   py::class_<SgmmPlan, std::shared_ptr<SgmmPlan>>(m, "SgmmPlan")
       .def_readonly("buf", &SgmmPlan::buf)
       .def_readonly("usable", &SgmmPlan::usable)
       .def_readonly("n_requests", &SgmmPlan::n_requests)
       .def_readonly("n_tokens", &SgmmPlan::n_tokens)
       .def_readonly("max_rank", &SgmmPlan::max_rank)
-      .def_readonly("max_input_len", &SgmmPlan::max_input_len);
+      .def_readonly("max_input_len", &SgmmPlan::max_input_len)
+      .def("status", [](const SgmmPlan& pl) { return plan_status_of(pl.buf); },
+           "status word of the plan (waits for the current stream): 0, or 1 = a launch of another shape was given "
+           "this plan and did nothing");
 
   m.def("slora_version", [] { return slora_version(); });
   m.def("dispatch_bgmv", &dispatch_bgmv, "dispatch_bgmv", py::arg("y"), py::arg("x"), py::arg("w"),

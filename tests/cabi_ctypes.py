@@ -40,6 +40,7 @@ SIGNATURES = {
     "slora_bgmv_expand_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _TP, _P, _P, _I, _I64, _I64, _I64, _I64, _I64,
                                    _I64, _I64, _I, _P]),
     "slora_bgmv_plan_bytes": (_I64, [_I64, _I64]),
+    "slora_plan_status": (_I, [_P, C.POINTER(C.c_int), _P]),
     "slora_bgmv_plan_build": (_I, [_P, _I64, _TP, _P, _I64, _I64, _I64, _P]),
     "slora_bgmv_shrink_planned": (_I, [_P, _I64, _I64, _I, _P, _P, _P, _P, _P, _TP, _P, _I64, _I64, _I64, _I64, _I64,
                                        _I, _I, _P]),

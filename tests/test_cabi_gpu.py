@@ -143,3 +143,47 @@ def test_prefill_operators_through_the_c_abi(hip, dtype):
         y_ref = O.ref_prefill_expand(np.zeros((T, H), np.float32), o_gpu, c.value, c.scales, c.a_loc, c.a_start,
                                      c.a_len, start, lens, ids, p, R, dtype)
         np.testing.assert_allclose(y_gpu, y_ref, rtol=RTOL, atol=ATOL)
+
+
+def test_a_plan_of_another_rank_cap_does_nothing_and_says_so(hip):
+    """A planned launch that names another rank cap or batch than the plan was built for leaves its
+    output alone and sets bit 0 of the plan's status word; the launch the plan was built for works
+    and the word is 0 after a build.  The buffer is sized for the largest launch made with it: a
+    launch reads its item records before it has seen the header."""
+    import cabi_ctypes as A
+    lib = A.load_library()
+    ranks = [16, 8, 32]
+    H, batch, R = 512, 9, 64
+    c = make_case(23, H, ranks, batch, dtype="f16")
+    key = hip.upload(to_bits(c.key, "f16"))
+    tables = A.SloraTables(hip.upload(c.a_start.astype(np.int64)), hip.upload(c.a_len.astype(np.int64)),
+                           hip.upload(c.a_loc.astype(np.int64)), len(ranks), int(c.a_loc.size))
+    bins = hip.upload(c.bins.astype(np.int64))
+    x = hip.upload(to_bits(c.x, "f16"))
+    nbytes = lib.slora_bgmv_plan_bytes(batch, R)
+    assert nbytes >= lib.slora_bgmv_plan_bytes(batch, 32) and nbytes >= lib.slora_bgmv_plan_bytes(batch - 1, R)
+    plan = hip.upload(np.zeros(nbytes // 4, np.int32))
+    status = C.c_int(-1)
+
+    def shrink(n_tokens, rank_cap, delta):
+        rc = lib.slora_bgmv_shrink_planned(plan, rank_cap, 0, 1, delta, None, None, x, key, C.byref(tables), bins,
+                                           n_tokens, H, R, c.page_elems, c.n_pages, 0, A.DTYPE_F16, None)
+        assert rc == A.OK, A.strerror(rc)
+
+    for what, n_tokens, rank_cap in (("rank cap", batch, 32), ("batch", batch - 1, R)):
+        assert lib.slora_bgmv_plan_build(plan, nbytes, C.byref(tables), bins, batch, R, c.n_pages, None) == A.OK
+        assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
+        delta = hip.upload(np.full((batch, R), 0x3c00, np.uint16))
+        print(f"c-abi planned shrink that names another {what}", flush=True)
+        shrink(n_tokens, rank_cap, delta)
+        assert np.all(hip.download(delta, (batch, R), np.uint16) == 0x3c00)
+        assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 1
+    # the launch the plan was built for
+    assert lib.slora_bgmv_plan_build(plan, nbytes, C.byref(tables), bins, batch, R, c.n_pages, None) == A.OK
+    delta = hip.upload(np.zeros((batch, R), np.uint16))
+    print("c-abi planned shrink with its own plan", flush=True)
+    shrink(batch, R, delta)
+    d_gpu = from_bits(hip.download(delta, (batch, R), np.uint16), "f16")
+    d_ref = O.ref_bgmv_shrink(np.zeros((batch, R), np.float32), c.x, c.key, c.a_start, c.a_len, c.a_loc, c.bins, 0, "f16")
+    np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
+    assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
