@@ -31,12 +31,12 @@ HBM_PEAK_GBS = 8000.0
 # a plain 256 MiB copy: 2.000 and 1.000); keyed by (workload, batch, mode, kernel).
 # None where not measured.
 TRAFFIC_BYTES = {
-    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true>"): 81522607,  # 75231151 read + 6291456 written
-    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70958584,  # the q/k/v launch
-    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 1>"): 281702660,  # 155676677 read + 126025983 written
-    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 3>"): 860963401,  # 482886010 read + 378077390 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16, 1, false>"): 142107743,  # 140138591 read + 1969152 written
-    ("c3", "sgmm_shrink_planned_kernel<BF16, 3, false>"): 174451508,  # 168544052 read + 5907456 written
+    ("s2", 256, "planned-fused", "bgmv_expand_kernel<F16, 3, true, 8>"): 81465122,  # 75173666 read + 6291456 written
+    ("s2", 256, "planned-fused", "bgmv_shrink_kernel<F16, true, 8>"): 70979806,  # the q/k/v launch
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 1>"): 281689745,  # 155663826 read + 126025919 written
+    ("c3", "sgmm_expand_walk_kernel<BF16, 2, 3>"): 860943997,  # 482866722 read + 378077275 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 1, false, true>"): 142557796,  # 140588644 read + 1969152 written
+    ("c3", "sgmm_shrink_planned_kernel<BF16, 3, false, true>"): 174280962,  # 168373506 read + 5907456 written
 }
 
 
