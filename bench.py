@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--batch", type=int, default=256)
-    ap.add_argument("--workload", choices=["s2", "s4", "s6", "c3", "load"], default="s2",
+    ap.add_argument("--workload", choices=["s2", "s4", "s6", "c3", "load", "streaming"], default="s2",
                     help="s2 (the metric's configuration), s4, s6: decode steps; c3: the prefill (segmented) kernels; "
                          "load: copying adapters into the pool; the last two are reported in the same format with "
                          "their own metric names")
@@ -695,6 +695,75 @@ def main_load(args, torch, device):
     print(json.dumps(out), flush=True)
 
 
+def main_streaming(args, torch, device):
+    """What plain reads of pool pages reach on this chip, with the library's own checksum kernel
+    (one wavefront per 8 KiB page, loads only; four pages per workgroup, consecutive workgroups
+    on consecutive XCDs): launches of several sizes over scattered pages (the fit t = t0 + bytes /
+    rate is the ceiling the decode launches are held against), one pool against one pool per
+    launch, and pages that are read twice -- by the same workgroup, by another workgroup of the
+    same XCD, by a workgroup of another XCD."""
+    import numpy as np
+    from slora_hip.infer_adapter import page_checksums
+    L, n_pages, page_elems = min(args.layers, 32), 65536, 4096
+    pools = [torch.zeros((n_pages, page_elems), dtype=torch.float16, device=device) for _ in range(L)]
+    rng = np.random.default_rng(0)
+    use_graph = args.launch == "graph"
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a).astype(np.int64)).to(device)
+
+    def timed(lists, pool_of):
+        def sweep():
+            for l in range(L):
+                page_checksums(pools[pool_of(l)], lists[l % len(lists)])
+        fn = graphed(sweep, torch) if use_graph else sweep
+        return time_region(fn, max(5, args.steps // 2), 3, torch) * 1e3 / L
+
+    def repeated(b, times, apart):
+        # blocks of `apart` entries, each block `times` times in a row: the copies of a page are `apart` entries apart
+        blocks = b[: len(b) // apart * apart].reshape(-1, apart)
+        return np.repeat(blocks[:, None, :], times, axis=1).reshape(-1)
+
+    page_bytes = page_elems * 2
+    sizes = {}
+    for n in (3072, 7944, 9728, 18432):   # 25, 65, 80, 151 MB per launch
+        lists = [dev(rng.permutation(n_pages)[:n]) for _ in range(4)]
+        us = timed(lists, lambda l: l)
+        sizes[n] = us
+    ns = np.array(sorted(sizes)); ts = np.array([sizes[n] for n in ns])
+    slope, t0 = np.polyfit(ns * page_bytes, ts, 1)      # us per byte, us
+    K = 7944
+    base = [rng.permutation(n_pages)[:K] for _ in range(4)]
+    uniq = [dev(b) for b in base]
+    rows = {
+        "one pool per launch (%d pools in turn)" % L: (K, timed(uniq, lambda l: l)),
+        "one pool for every launch": (K, timed(uniq, lambda l: 0)),
+        "each page twice, same workgroup": (2 * K, timed([dev(repeated(b, 2, 1)) for b in base], lambda l: l)),
+        "each page twice, next workgroup of the same XCD": (2 * (K // 32 * 32),
+                                                            timed([dev(repeated(b, 2, 32)) for b in base], lambda l: l)),
+        "each page twice, next workgroup (another XCD)": (2 * K, timed([dev(repeated(b, 2, 4)) for b in base], lambda l: l)),
+        "twice as many different pages": (2 * K, timed([dev(rng.permutation(n_pages)[:2 * K]) for _ in range(4)],
+                                                       lambda l: l)),
+    }
+    rate = 1.0 / slope / 1e3   # GB/s
+    out = {
+        "metric": "read-only streaming of scattered pool pages, asymptotic GB/s",
+        "value": round(rate, 1), "unit": "GB/s", "n_gpus": 1, "steps": max(5, args.steps // 2), "warmup": 3,
+        "ms_per_step": round(sizes[7944] * L * 1e-3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"page checksums over {L} pools of {n_pages} pages of {page_bytes} bytes",
+                   "launch": args.launch},
+        "roofline": {"kernel": "page_xor_kernel", "bound": "hbm", "achieved": round(rate, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(rate / HBM_PEAK_GBS, 4), "traffic": None},
+        "launch_sizes": {"us_per_launch_by_pages": {str(n): round(sizes[n], 3) for n in ns},
+                         "fit": {"fixed_us": round(float(t0), 3), "GBps": round(rate, 1)}},
+        "reads_of_%d_pages" % K: {k: {"page_reads": n, "us_per_launch": round(us, 3),
+                                      "GBps_of_page_reads": round(n * page_bytes / us / 1e3, 1)}
+                                  for k, (n, us) in rows.items()},
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -722,6 +791,9 @@ def main():
         return
     if args.workload == "load":
         main_load(args, torch, device)
+        return
+    if args.workload == "streaming":
+        main_streaming(args, torch, device)
         return
     if args.workload == "s2":
         w = workloads.s2_decode(device, n_layers=args.layers, batch=args.batch, placement=args.placement)
