@@ -196,7 +196,7 @@ def test_bmm_equals_dense_f64_and_paged():
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_16bit_paths_within_stated_tolerance_of_bmm(dtype):
-    """BASELINE tolerance (rtol 1e-2, atol 1e-3... scaled by the bf16 epsilon
+    """The stated tolerance (rtol 1e-2, atol 1e-3... scaled by the bf16 epsilon
     for bf16, see the GPU tests) between the paged and the bmm rounding chains."""
     c = make_case(21, 256, [8, 16, 64], batch=16, dtype=dtype)
     p = 0
