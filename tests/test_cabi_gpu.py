@@ -187,3 +187,50 @@ def test_a_plan_of_another_rank_cap_does_nothing_and_says_so(hip):
     d_ref = O.ref_bgmv_shrink(np.zeros((batch, R), np.float32), c.x, c.key, c.a_start, c.a_len, c.a_loc, c.bins, 0, "f16")
     np.testing.assert_allclose(d_gpu, d_ref, rtol=RTOL, atol=ATOL)
     assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
+
+
+def test_a_prefill_plan_of_another_batch_does_nothing_and_says_so(hip):
+    """slora_sgmm_shrink_planned with the plan of another batch shape leaves its output alone and sets
+    the plan's status word; with its own plan it gives the oracle's result and the word is 0."""
+    import cabi_ctypes as A
+    lib = A.load_library()
+    ranks = [64, 16, 8, 32]
+    H, R, dtype = 512, 64, "f16"
+    start, lens, ids = make_segments(5, 6, 20, 90, len(ranks))
+    T = int(lens.sum())
+    c = make_case(24, H, ranks, T, dtype=dtype, bins=np.repeat(ids, lens))
+    key = hip.upload(to_bits(c.key, dtype))
+    tables = A.SloraTables(hip.upload(c.a_start.astype(np.int64)), hip.upload(c.a_len.astype(np.int64)),
+                           hip.upload(c.a_loc.astype(np.int64)), len(ranks), int(c.a_loc.size))
+    st, ln, rq = hip.upload(start.astype(np.int32)), hip.upload(lens.astype(np.int32)), hip.upload(ids.astype(np.int64))
+    x = hip.upload(to_bits(c.x, dtype))
+    nbytes = lib.slora_sgmm_plan_bytes()
+    plan = hip.upload(np.zeros(nbytes // 4, np.int32))
+    usable, status = C.c_int(0), C.c_int(-1)
+
+    def build(n_req, max_len, n_tokens):
+        rc = lib.slora_sgmm_plan_build(plan, nbytes, C.byref(tables), st, ln, rq, n_req, max_len, n_tokens, R,
+                                       C.byref(usable), None)
+        assert rc == A.OK and usable.value == 1
+
+    def shrink(o):
+        return lib.slora_sgmm_shrink_planned(plan, o, x, key, C.byref(tables), st, ln, rq, len(lens), int(lens.max()), T, H,
+                                             R, H, H, R, c.n_pages, 0, A.DTYPE_F16, None)
+
+    # a plan for the first request alone: another number of row parts than the launch below has
+    build(1, int(lens[0]), int(lens[0]))
+    assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
+    o = hip.upload(np.full((T, R), 0x3c00, np.uint16))
+    print("c-abi planned prefill shrink with the plan of another batch", flush=True)
+    assert shrink(o) == A.OK
+    assert np.all(hip.download(o, (T, R), np.uint16) == 0x3c00)
+    assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 1
+    build(len(lens), int(lens.max()), T)
+    assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
+    print("c-abi planned prefill shrink with its own plan", flush=True)
+    assert shrink(o) == A.OK
+    o_gpu = from_bits(hip.download(o, (T, R), np.uint16), dtype)
+    o_ref = O.ref_prefill_shrink(np.ones((T, R), np.float32), c.x, c.key, c.a_loc, c.a_start, c.a_len, start, lens, ids,
+                                 0, R, dtype)
+    np.testing.assert_allclose(o_gpu, o_ref, rtol=RTOL, atol=ATOL)
+    assert lib.slora_plan_status(plan, C.byref(status), None) == A.OK and status.value == 0
