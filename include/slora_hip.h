@@ -155,7 +155,8 @@ SLORA_API int slora_bgmv_plan_build(void* plan, int64_t plan_bytes, const slora_
  * abandoned after its poll limit.  The mark covers a wrong plan in a large enough buffer only: a
  * planned launch reads its item records before it has seen the header, so the buffer it is given
  * must hold slora_bgmv_plan_bytes(batch, rank_cap) bytes for the batch and rank cap OF THE LAUNCH,
- * whatever the plan in it was built for.  No counterpart in the reference. */
+ * whatever the plan in it was built for.  Not to be called on a stream that is being captured
+ * into a graph (it copies to the host and waits).  No counterpart in the reference. */
 SLORA_API int slora_plan_status(const void* plan, int* status, void* stream);
 
 /* slora_bgmv_shrink / slora_bgmv_shrink_qkv with a plan.  nproj = 1: y0 and
