@@ -738,6 +738,8 @@ def main_streaming(args, torch, device):
     rows = {
         "one pool per launch (%d pools in turn)" % L: (K, timed(uniq, lambda l: l)),
         "one pool for every launch": (K, timed(uniq, lambda l: 0)),
+        "the same pages in every launch (65 MB, warm in the 256 MB Infinity Cache)": (K, timed(uniq[:1], lambda l: 0)),
+        "the same pages in every second launch": (K, timed(uniq[:2], lambda l: 0)),
         "each page twice, same workgroup": (2 * K, timed([dev(repeated(b, 2, 1)) for b in base], lambda l: l)),
         "each page twice, next workgroup of the same XCD": (2 * (K // 32 * 32),
                                                             timed([dev(repeated(b, 2, 32)) for b in base], lambda l: l)),
